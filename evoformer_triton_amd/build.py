@@ -1,0 +1,82 @@
+"""Builds libevoattn.so (gfx950) in-tree with hipcc.
+
+    python -m evoformer_triton_amd.build [--force]
+
+One object per (kernel file, head dim) so that the objects compile in parallel; the result
+is evoformer_triton_amd/libevoattn.so, a plain C-ABI library (include/evoattn.h) that links
+against the HIP runtime only.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libevoattn.so")
+HEAD_DIMS = (8, 16, 32, 64)
+
+# -packed-fp32-ops off: packed fp32 VALU forms are not used on this hardware pool.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+]
+
+
+def _units():
+    units = [("api", "api.hip", []), ("generic", "generic.hip", []), ("dispatch", "dispatch.hip", [])]
+    for d in HEAD_DIMS:
+        units.append((f"mfma_fwd_d{d}", "mfma_fwd.hip", [f"-DEVO_D={d}"]))
+        units.append((f"mfma_bwd_d{d}", "mfma_bwd.hip", [f"-DEVO_D={d}"]))
+    return units
+
+
+def _hipcc():
+    for c in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if c and (os.path.sep not in c or os.path.exists(c)):
+            return c
+    raise RuntimeError("hipcc not found")
+
+
+def _compile(unit):
+    name, src, defs = unit
+    out = os.path.join(OBJ, name + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {name}:\n{err}")
+    return out, err
+
+
+def build(force: bool = True, verbose: bool = False, jobs: int | None = None) -> str:
+    """Compile every HIP source for gfx950 and link the shared library."""
+    os.makedirs(OBJ, exist_ok=True)
+    units = _units()
+    if not force and os.path.exists(LIB):
+        newest = max(os.path.getmtime(os.path.join(r, f)) for r, _, fs in os.walk(CSRC) for f in fs)
+        newest = max(newest, os.path.getmtime(os.path.join(ROOT, "include", "evoattn.h")))
+        if os.path.getmtime(LIB) >= newest:
+            return LIB
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        results = list(ex.map(_compile, units))
+    if verbose:
+        for _, err in results:
+            if err.strip():
+                print(err, file=sys.stderr)
+    objs = [o for o, _ in results]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv or True, verbose=True))

@@ -1,0 +1,180 @@
+// C ABI of the library: parameter validation, workspace layout and kernel dispatch.
+// Everything in this file runs on the host; nothing here needs a GPU except the two
+// enqueue entry points.
+#include "common.h"
+#include "kernels.h"
+
+namespace evo {
+
+static inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+static inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
+static inline int elem_size(int dtype) { return dtype == EVO_F32 ? 4 : 2; }
+
+static int check_common(const EvoAttnParams *p) {
+    if (!p) return EVO_EINVAL;
+    if (p->B <= 0 || p->S <= 0 || p->N <= 0 || p->H <= 0 || p->D <= 0) return EVO_EINVAL;
+    if (p->dtype != EVO_BF16 && p->dtype != EVO_F16 && p->dtype != EVO_F32) return EVO_EINVAL;
+    if (p->bias_dtype != EVO_NONE && p->bias_dtype != EVO_F32 && p->bias_dtype != p->dtype) return EVO_EINVAL;
+    if (p->mask_kind < EVO_MASK_NONE || p->mask_kind > EVO_MASK_F16) return EVO_EINVAL;
+    if ((p->bias_dtype == EVO_NONE) != (p->bias == nullptr)) return EVO_EINVAL;
+    if ((p->mask_kind == EVO_MASK_NONE) != (p->mask == nullptr)) return EVO_EINVAL;
+    if (!p->q || !p->k || !p->v || !p->o || !p->lse) return EVO_EINVAL;
+    if (!(p->scale == p->scale) || p->scale <= 0.0f) return EVO_EINVAL;
+    if (p->D != 8 && p->D != 16 && p->D != 32 && p->D != 64 && p->D != 128) return EVO_EUNSUPPORTED;
+    if (p->stride_b < 0 || p->stride_h < 0 || p->stride_s < 0 || p->stride_n < p->D) return EVO_EINVAL;
+    if (p->bias && (p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_row < p->N)) return EVO_EINVAL;
+    if (p->mask && (p->mask_stride_b < 0 || p->mask_stride_s < 0)) return EVO_EINVAL;
+    // index ranges: problems and rows are 32-bit in the kernels, element offsets 64-bit
+    const int64_t probs = (int64_t)p->B * p->H * p->S;
+    if (probs > (int64_t)1 << 26 || (int64_t)p->N > (int64_t)1 << 20) return EVO_EOVERFLOW;
+    if (probs * ((p->N + 31) / 32) > (int64_t)0x7fffffff) return EVO_EOVERFLOW;
+    if ((int64_t)p->B * p->H * p->N * ((p->N + 63) / 64) > (int64_t)0x7fffffff) return EVO_EOVERFLOW;
+    const int es = elem_size(p->dtype);
+    if (!aligned(p->q, es) || !aligned(p->k, es) || !aligned(p->v, es) || !aligned(p->o, es) || !aligned(p->lse, 4))
+        return EVO_EALIGN;
+    if (p->bias && !aligned(p->bias, elem_size(p->bias_dtype))) return EVO_EALIGN;
+    if (p->mask_kind == EVO_MASK_F32 && !aligned(p->mask, 4)) return EVO_EALIGN;
+    if ((p->mask_kind == EVO_MASK_BF16 || p->mask_kind == EVO_MASK_F16) && !aligned(p->mask, 2)) return EVO_EALIGN;
+    return EVO_OK;
+}
+
+// The matrix-core kernels read rows with 16-byte loads and keep one 32-wide key tile per
+// 16 accumulator registers in the dBias kernel (at most 16 tiles per wave, 4 waves).
+static bool mfma_ok(const EvoAttnParams &p, int pass) {
+    if (p.flags & EVO_FLAG_FORCE_GENERIC) return false;
+    if (p.dtype != EVO_BF16 && p.dtype != EVO_F16) return false;
+    if (p.D != 8 && p.D != 16 && p.D != 32 && p.D != 64) return false;
+    if (p.stride_b % 8 || p.stride_h % 8 || p.stride_s % 8 || p.stride_n % 8) return false;
+    if (!aligned(p.q, 16) || !aligned(p.k, 16) || !aligned(p.v, 16) || !aligned(p.o, 16)) return false;
+    if (pass == EVO_PASS_BWD) {
+        if (p.N > 2048) return false;
+        if (!aligned(p.dout, 16) || !aligned(p.dq, 16) || !aligned(p.dk, 16) || !aligned(p.dv, 16)) return false;
+    }
+    return true;
+}
+
+static int bias_vec_ok(const EvoAttnParams &p) {
+    if (!p.bias) return 0;
+    const size_t a = p.bias_dtype == EVO_F32 ? 16 : 8;
+    return aligned(p.bias, a) && p.bias_stride_b % 4 == 0 && p.bias_stride_h % 4 == 0 && p.bias_stride_row % 4 == 0;
+}
+
+// S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
+// writes one partial dBias tile.  Enough chunks to fill the chip, no more.
+static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
+    const int64_t base = (int64_t)((p.N + 31) / 32) * p.B * p.H;
+    int64_t want = (1024 + base - 1) / base;
+    if (want < 1) want = 1;
+    if (want > p.S) want = p.S;
+    *chunk = (int)((p.S + want - 1) / want);
+    *n_chunks = (p.S + *chunk - 1) / *chunk;
+}
+
+struct WsLayout {
+    size_t delta, shift, dmask_part, dbias_part, total;
+    int n_chunks, chunk;
+};
+
+static WsLayout ws_layout(const EvoAttnParams &p) {
+    WsLayout w{};
+    const size_t rows = (size_t)p.B * p.H * p.S * p.N;
+    size_t off = 0;
+    w.delta = off; off += align_up(rows * 4);
+    w.shift = off; off += align_up((size_t)p.B * p.S * 4);
+    w.dmask_part = off; if (p.dmask) off += align_up(rows * 4);
+    chunking(p, &w.n_chunks, &w.chunk);
+    w.dbias_part = off;
+    if (p.dbias) off += align_up((size_t)w.n_chunks * p.B * p.H * p.N * p.N * 4);
+    w.total = off;
+    return w;
+}
+
+static int check_bwd(const EvoAttnParams *p) {
+    if (!p->dout || !p->dq || !p->dk || !p->dv) return EVO_EINVAL;
+    const int es = elem_size(p->dtype);
+    if (!aligned(p->dout, es) || !aligned(p->dq, es) || !aligned(p->dk, es) || !aligned(p->dv, es)) return EVO_EALIGN;
+    if (p->dbias) {
+        if (p->dbias_dtype != EVO_F32 && p->dbias_dtype != p->dtype) return EVO_EINVAL;
+        if (!aligned(p->dbias, elem_size(p->dbias_dtype))) return EVO_EALIGN;
+    }
+    if (p->dmask && !aligned(p->dmask, 4)) return EVO_EALIGN;
+    const WsLayout w = ws_layout(*p);
+    if (!p->workspace || p->workspace_bytes < w.total) return EVO_EWORKSPACE;
+    if (!aligned(p->workspace, 256)) return EVO_EALIGN;
+    return EVO_OK;
+}
+
+}  // namespace evo
+
+using namespace evo;
+
+extern "C" {
+
+int evoattn_version(void) { return EVOATTN_VERSION; }
+
+const char *evoattn_strerror(int code) {
+    switch (code) {
+        case EVO_OK: return "ok";
+        case EVO_EINVAL: return "invalid argument (null pointer, non-positive size or bad enum)";
+        case EVO_EUNSUPPORTED: return "unsupported head dimension or size";
+        case EVO_EALIGN: return "pointer or stride not aligned for the dtype";
+        case EVO_EWORKSPACE: return "workspace missing or too small";
+        case EVO_EOVERFLOW: return "extents overflow the kernels' index range";
+    }
+    if (code <= EVO_EHIP) return hipGetErrorString((hipError_t)(EVO_EHIP - code));
+    return "unknown error";
+}
+
+int evoattn_check(const EvoAttnParams *p, int pass) {
+    int rc = check_common(p);
+    if (rc) return rc;
+    if (pass == EVO_PASS_BWD) return check_bwd(p);
+    if (pass != EVO_PASS_FWD) return EVO_EINVAL;
+    return EVO_OK;
+}
+
+size_t evoattn_bwd_workspace_bytes(const EvoAttnParams *p) {
+    if (!p || p->B <= 0 || p->S <= 0 || p->N <= 0 || p->H <= 0) return 0;
+    return ws_layout(*p).total;
+}
+
+const char *evoattn_path(const EvoAttnParams *p, int pass) {
+    if (!p) return "invalid";
+    return mfma_ok(*p, pass) ? "mfma" : "generic";
+}
+
+int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
+    int rc = evoattn_check(p, EVO_PASS_FWD);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)hip_stream;
+    if (!mfma_ok(*p, EVO_PASS_FWD)) return launch_generic_fwd(*p, st);
+    Extra e{};
+    e.vec_ok = bias_vec_ok(*p);
+    return launch_mfma_fwd(*p, e, st);
+}
+
+int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
+    int rc = evoattn_check(p, EVO_PASS_BWD);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)hip_stream;
+    const WsLayout w = ws_layout(*p);
+    char *ws = (char *)p->workspace;
+    Extra e{};
+    e.n_chunks = w.n_chunks;
+    e.chunk = w.chunk;
+    e.vec_ok = bias_vec_ok(*p);
+    e.delta = (float *)(ws + w.delta);
+    e.shift = (float *)(ws + w.shift);
+    e.dmask_part = (float *)(ws + w.dmask_part);
+    e.dbias_part = (float *)(ws + w.dbias_part);
+    if (!mfma_ok(*p, EVO_PASS_BWD)) return launch_generic_bwd(*p, e, st);
+    if ((rc = launch_mfma_delta(*p, e, st))) return rc;
+    if ((rc = launch_mask_shift(*p, e, st))) return rc;
+    if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;
+    if ((rc = launch_mfma_dq(*p, e, st))) return rc;
+    if (p->dbias && (rc = launch_dbias_reduce(*p, e, st))) return rc;
+    if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;
+    return EVO_OK;
+}
+
+}  // extern "C"

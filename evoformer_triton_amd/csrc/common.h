@@ -1,0 +1,181 @@
+// Shared device/host helpers for the gfx950 Evoformer attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <float.h>
+#include <stdint.h>
+
+#include "evoattn.h"
+
+#define EVO_CAT_(a, b) a##b
+#define EVO_CAT(a, b) EVO_CAT_(a, b)
+
+namespace evo {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+// A problem whose every key has a mask value below this is shifted by its largest mask
+// value so that the log-sum-exp keeps its mantissa.
+constexpr float kShiftThreshold = -1.0e4f;
+
+// Launch-time constants derived on the host.
+struct Extra {
+    int n_chunks;      // number of S-chunks the dBias partials are split into
+    int chunk;         // rows of S per chunk
+    int vec_ok;        // bias rows may be read with 8/16-byte vector loads
+    float *delta;      // [B][H][S][N]
+    float *shift;      // [B][S] per-row mask shift
+    float *dbias_part; // [n_chunks][B][H][N][N]
+    float *dmask_part; // [B][H][S][N]
+};
+
+// Linear block id -> logical id such that consecutive logical ids run on one XCD
+// (hardware deals consecutive workgroup ids round-robin over the 8 XCDs, each with its
+// own L2).  Bijection on [0,total) for any total.
+__device__ __forceinline__ unsigned xcd_remap(unsigned id, unsigned total) {
+    constexpr unsigned X = 8;
+    unsigned x = id % X, slot = id / X;
+    unsigned q = total / X, r = total % X;
+    return x * q + (x < r ? x : r) + slot;
+}
+
+struct Prob {
+    int b, h, s;
+    int64_t base;  // element offset of row 0 in the q-family tensors
+    int64_t row0;  // offset of row 0 in lse / delta
+};
+
+__device__ __forceinline__ Prob decode_problem(const EvoAttnParams &p, unsigned pid) {
+    Prob r;
+    r.s = pid % p.S;
+    unsigned t = pid / p.S;
+    r.h = t % p.H;
+    r.b = t / p.H;
+    r.base = (int64_t)r.b * p.stride_b + (int64_t)r.h * p.stride_h + (int64_t)r.s * p.stride_s;
+    r.row0 = (int64_t)pid * p.N;
+    return r;
+}
+
+// Additive form of mask[b][s][key]; -inf past the end of the row so that padded keys get
+// zero probability whatever the rest of the row holds.
+__device__ __forceinline__ float mask_add(const EvoAttnParams &p, int b, int s, int key) {
+    if (key >= p.N) return -INFINITY;
+    if (p.mask_kind == EVO_MASK_NONE) return 0.0f;
+    int64_t off = (int64_t)b * p.mask_stride_b + (int64_t)s * p.mask_stride_s + key;
+    switch (p.mask_kind) {
+        case EVO_MASK_BOOL: return ((const uint8_t *)p.mask)[off] ? 0.0f : -FLT_MAX;
+        case EVO_MASK_F32:  return ((const float *)p.mask)[off];
+        case EVO_MASK_BF16: return (float)((const bf16_t *)p.mask)[off];
+        default:            return (float)((const f16_t *)p.mask)[off];
+    }
+}
+
+__device__ __forceinline__ float shift_from_max(float mx) { return mx < kShiftThreshold ? fmaxf(mx, -FLT_MAX) : 0.0f; }
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <typename T> struct Mfma;
+template <> struct Mfma<bf16_t> {
+    typedef bf16x8 v8;
+    typedef bf16x4 v4;
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ f32x16 mma(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mfma<f16_t> {
+    typedef f16x8 v8;
+    typedef f16x4 v4;
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ f32x16 mma(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// 32x32x16 MFMA operand / accumulator geometry used by every kernel (lane l, g = l / 32):
+//   A (32 x 16): lane holds row l % 32, columns 8g .. 8g+7
+//   B (16 x 32): lane holds column l % 32, rows 8g .. 8g+7
+//   C (32 x 32): lane holds column l % 32, register r holds row 8*(r/4) + 4g + r%4
+// A C tile is fed back as a B operand without any cross-lane traffic: k-step t takes
+// registers 8t .. 8t+7, whose rows are crow(8t+i, g); the matching A operand must then list
+// its columns in that row order, which acol_pos() gives as a storage position.
+__device__ __forceinline__ int crow(int r, int g) { return 8 * (r >> 2) + 4 * g + (r & 3); }
+// position, inside a run of 32, at which row/key `x` is stored so that the 8 values one
+// lane group needs for one k-step are contiguous: x = 16t + 8u + 4g + i -> 16t + 8g + 4u + i
+__device__ __forceinline__ int perm_pos(int x) {
+    return (x & ~15) | ((x & 4) << 1) | ((x & 8) >> 1) | (x & 3);
+}
+
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 ld8(const T *ptr) {
+    return *reinterpret_cast<const typename Mfma<T>::v8 *>(ptr);
+}
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 zero8() {
+    typename Mfma<T>::v8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = (T)0.0f;
+    return z;
+}
+
+// Four bias values for one query row and four consecutive keys, as fp32.
+// BIASK: 0 none, 1 fp32, 2 same 16-bit type as T.
+template <int BIASK, typename T>
+__device__ __forceinline__ void load_bias4(const void *bias, int64_t off, int nvalid, bool vec, float out[4]) {
+    if (BIASK == 0) {
+        out[0] = out[1] = out[2] = out[3] = 0.0f;
+    } else if (BIASK == 1) {
+        const float *b = (const float *)bias + off;
+        if (vec && nvalid >= 4) {
+            f32x4 v = *reinterpret_cast<const f32x4 *>(b);
+            out[0] = v[0]; out[1] = v[1]; out[2] = v[2]; out[3] = v[3];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = i < nvalid ? b[i] : 0.0f;
+        }
+    } else {
+        const T *b = (const T *)bias + off;
+        if (vec && nvalid >= 4) {
+            typename Mfma<T>::v4 v = *reinterpret_cast<const typename Mfma<T>::v4 *>(b);
+            out[0] = (float)v[0]; out[1] = (float)v[1]; out[2] = (float)v[2]; out[3] = (float)v[3];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[i] = i < nvalid ? (float)b[i] : 0.0f;
+        }
+    }
+}
+
+template <int BIASK, typename T>
+__device__ __forceinline__ float load_bias1(const void *bias, int64_t off) {
+    if (BIASK == 0) return 0.0f;
+    if (BIASK == 1) return ((const float *)bias)[off];
+    return (float)((const T *)bias)[off];
+}
+
+// Store four consecutive fp32 values as T (8 bytes for 16-bit types).
+template <typename T>
+__device__ __forceinline__ void store4(T *dst, float a, float b, float c, float d) {
+    typename Mfma<T>::v4 v;
+    v[0] = (T)a; v[1] = (T)b; v[2] = (T)c; v[3] = (T)d;
+    *reinterpret_cast<typename Mfma<T>::v4 *>(dst) = v;
+}
+
+}  // namespace evo

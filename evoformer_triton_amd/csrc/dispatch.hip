@@ -1,0 +1,34 @@
+// Routes the matrix-core launches to the translation unit compiled for the head dim.
+#include "common.h"
+#include "kernels.h"
+
+namespace evo {
+
+#define EVO_DECL(D)                                                                          \
+    int launch_mfma_fwd_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
+    int launch_mfma_delta_d##D(const EvoAttnParams &, const Extra &, hipStream_t);           \
+    int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
+    int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
+EVO_DECL(8)
+EVO_DECL(16)
+EVO_DECL(32)
+EVO_DECL(64)
+#undef EVO_DECL
+
+#define EVO_ROUTE(name)                                                       \
+    int launch_mfma_##name(const EvoAttnParams &p, const Extra &e, hipStream_t st) { \
+        switch (p.D) {                                                        \
+            case 8: return launch_mfma_##name##_d8(p, e, st);                 \
+            case 16: return launch_mfma_##name##_d16(p, e, st);               \
+            case 32: return launch_mfma_##name##_d32(p, e, st);               \
+            case 64: return launch_mfma_##name##_d64(p, e, st);               \
+        }                                                                     \
+        return EVO_EUNSUPPORTED;                                              \
+    }
+EVO_ROUTE(fwd)
+EVO_ROUTE(delta)
+EVO_ROUTE(dq)
+EVO_ROUTE(dkdv)
+#undef EVO_ROUTE
+
+}  // namespace evo

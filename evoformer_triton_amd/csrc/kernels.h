@@ -1,0 +1,21 @@
+// Host-side launchers of the kernel families; each enqueues on `st` and returns EVO_OK or
+// EVO_EHIP - hipError_t.
+#pragma once
+
+#include "common.h"
+
+namespace evo {
+
+int launch_generic_fwd(const EvoAttnParams &p, hipStream_t st);
+int launch_generic_bwd(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_delta_generic(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_dmask_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_dbias_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_mask_shift(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+
+int launch_mfma_fwd(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_mfma_delta(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_mfma_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_mfma_dkdv(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+
+}  // namespace evo

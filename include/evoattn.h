@@ -1,0 +1,133 @@
+/*
+ * evoattn.h - C ABI of the MI355X (gfx950) Evoformer attention library.
+ *
+ * One attention "problem" is (b, h, s): N query rows against N key rows of width D,
+ *     O = softmax(scale * Q K^T + pair_bias[b,h] + row_mask[b,s]) V.
+ * The library holds the device kernels the reference generates with Triton; the host
+ * (a torch.autograd.Function, a C++ trainer, ...) owns every buffer, hands in raw device
+ * pointers, element strides and a HIP stream.  No entry point allocates, synchronises,
+ * throws or touches any stream but the one it is given.  All return 0 or a negative
+ * EVO_E* code; evoattn_strerror() names it.
+ *
+ * Reference interface each entry point stands in for (lvhoaa/evoformer_triton,
+ * dsevoformer-triton/evoformer.py):
+ *   evoattn_fwd  <- the `_attn_fwd[grid](...)` launch in EvoformerAttention.forward
+ *                   (evoformer.py:676-724; kernels :23-297)
+ *   evoattn_bwd  <- the three launches in EvoformerAttention.backward:
+ *                   `_attn_bwd_preprocess` (:761-768), `_attn_bwd_dk_dv` (:776-812),
+ *                   `_attn_bwd_dq` (:815-854), plus the zero-fill and the cast of
+ *                   d_pair_bias (:752, :860)
+ *   evoattn_bwd_workspace_bytes <- the `D = torch.empty_like(M)` and fp32 `d_pair_bias`
+ *                   staging allocations (:752, :758), sized for the caller to make
+ *   evoattn_check <- the asserts at :642-643 and :747-748
+ */
+#ifndef EVOATTN_H
+#define EVOATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EVOATTN_VERSION 1
+
+/* element types */
+enum {
+    EVO_NONE = -1,
+    EVO_BF16 = 0,
+    EVO_F16  = 1,
+    EVO_F32  = 2   /* "check mode": every product and sum in fp32, no matrix cores */
+};
+
+/* row-mask encodings; mask is indexed [b][s][key], key contiguous */
+enum {
+    EVO_MASK_NONE = 0,
+    EVO_MASK_BOOL = 1,  /* uint8, non-zero = keep; dropped keys score -FLT_MAX (evoformer.py:69) */
+    EVO_MASK_F32  = 2,  /* additive */
+    EVO_MASK_BF16 = 3,  /* additive */
+    EVO_MASK_F16  = 4   /* additive */
+};
+
+/* flags */
+enum {
+    EVO_FLAG_FORCE_GENERIC = 1  /* run the plain fp32-arithmetic kernels whatever the dtype */
+};
+
+/* error codes */
+enum {
+    EVO_OK            = 0,
+    EVO_EINVAL        = -1,  /* null pointer, non-positive size, bad enum */
+    EVO_EUNSUPPORTED  = -2,  /* head dim or size outside what the kernels cover */
+    EVO_EALIGN        = -3,  /* pointer or stride not aligned for the requested dtype */
+    EVO_EWORKSPACE    = -4,  /* workspace missing or too small */
+    EVO_EOVERFLOW     = -5,  /* extents overflow the index type */
+    EVO_EHIP          = -100 /* EVO_EHIP - hipError_t from a launch */
+};
+
+enum { EVO_PASS_FWD = 0, EVO_PASS_BWD = 1 };
+
+/*
+ * Strides are in elements.  q, k, v, o, dout, dq, dk, dv all share one stride set:
+ * element (b,h,s,n,d) lives at b*stride_b + h*stride_h + s*stride_s + n*stride_n + d.
+ * The reference's flat reinterpretation of a dense [B,S,N,H,D] tensor as [B,H,S,N,D]
+ * (evoformer.py:648-650) is (S*N*H*D, S*N*D, N*D, D); a true per-head view of the same
+ * tensor is (S*N*H*D, D, N*H*D, H*D).
+ * lse is dense [B][H][S][N] fp32.  For a problem whose every key carries a mask value
+ * below -1e4 the kernels subtract the largest mask value of the row from the scores
+ * before the softmax (it cancels in O and in every gradient) and lse holds the
+ * log-sum-exp of the shifted scores; otherwise lse = log sum_j exp(score_ij).
+ */
+typedef struct EvoAttnParams {
+    int32_t B, S, N, H, D;
+    int32_t dtype;        /* EVO_BF16 / EVO_F16 / EVO_F32 : q,k,v,o,dout,dq,dk,dv */
+    int32_t bias_dtype;   /* EVO_NONE, EVO_F32, or equal to dtype */
+    int32_t mask_kind;    /* EVO_MASK_* */
+    int32_t dbias_dtype;  /* dtype of dbias: EVO_F32 or equal to dtype (ignored if dbias NULL) */
+    int32_t flags;        /* EVO_FLAG_* */
+    float   scale;        /* softmax scale, normally D^-0.5 (evoformer.py:646) */
+    int32_t reserved;
+
+    int64_t stride_b, stride_h, stride_s, stride_n;          /* q-family */
+    int64_t bias_stride_b, bias_stride_h, bias_stride_row;    /* bias[b][h][row][col], col contiguous */
+    int64_t mask_stride_b, mask_stride_s;                     /* mask[b][s][key], key contiguous */
+
+    const void *q, *k, *v;
+    const void *bias;     /* may be NULL (bias_dtype = EVO_NONE) */
+    const void *mask;     /* may be NULL (mask_kind = EVO_MASK_NONE) */
+    void       *o;        /* fwd: out; bwd: in */
+    float      *lse;      /* fwd: out; bwd: in */
+
+    const void *dout;     /* bwd only below */
+    void       *dq, *dk, *dv;
+    void       *dbias;    /* dense [B][H][N][N], may be NULL */
+    float      *dmask;    /* dense [B][S][N] fp32 gradient of an additive mask, may be NULL */
+    void       *workspace;
+    size_t      workspace_bytes;
+} EvoAttnParams;
+
+int         evoattn_version(void);
+const char *evoattn_strerror(int code);
+
+/* Host-only validation of a parameter block for one pass; launches nothing. */
+int evoattn_check(const EvoAttnParams *p, int pass);
+
+/* Bytes of device workspace evoattn_bwd needs for this problem (0 on invalid input). */
+size_t evoattn_bwd_workspace_bytes(const EvoAttnParams *p);
+
+/* Enqueue the forward: writes o and lse. */
+int evoattn_fwd(const EvoAttnParams *p, void *hip_stream);
+
+/* Enqueue the backward: writes dq, dk, dv and, when non-NULL, dbias and dmask.
+ * Deterministic: no floating-point atomics; two runs give bit-identical results. */
+int evoattn_bwd(const EvoAttnParams *p, void *hip_stream);
+
+/* Name of the kernel family evoattn_fwd/evoattn_bwd would run for these parameters
+ * ("mfma" or "generic"); for tests and reports. */
+const char *evoattn_path(const EvoAttnParams *p, int pass);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EVOATTN_H */
