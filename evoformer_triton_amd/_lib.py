@@ -15,10 +15,11 @@ LIB_PATH = os.path.join(HERE, "libevoattn.so")
 EVO_NONE, EVO_BF16, EVO_F16, EVO_F32 = -1, 0, 1, 2
 EVO_MASK_NONE, EVO_MASK_BOOL, EVO_MASK_F32, EVO_MASK_BF16, EVO_MASK_F16 = 0, 1, 2, 3, 4
 EVO_FLAG_FORCE_GENERIC = 1
+EVO_FLAG_PREP_VALID = 2
 EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 
-EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_bwd_workspace_bytes",
+EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_prep_bytes", "evoattn_bwd_workspace_bytes",
            "evoattn_fwd", "evoattn_bwd", "evoattn_path")
 
 
@@ -39,6 +40,7 @@ class EvoAttnParams(ctypes.Structure):
         ("dout", ctypes.c_void_p), ("dq", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p),
         ("dbias", ctypes.c_void_p), ("dmask", ctypes.c_void_p),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("prep", ctypes.c_void_p), ("prep_bytes", ctypes.c_size_t),
     ]
 
 
@@ -69,6 +71,8 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_strerror.argtypes = [ctypes.c_int]
     lib.evoattn_check.restype = ctypes.c_int
     lib.evoattn_check.argtypes = [P, ctypes.c_int]
+    lib.evoattn_prep_bytes.restype = ctypes.c_size_t
+    lib.evoattn_prep_bytes.argtypes = [P]
     lib.evoattn_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.evoattn_bwd_workspace_bytes.argtypes = [P]
     lib.evoattn_fwd.restype = ctypes.c_int

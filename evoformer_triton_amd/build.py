@@ -28,11 +28,18 @@ HIPCC_FLAGS = [
 ]
 
 
+# Keep matrix-core accumulators in ordinary vector registers: the softmax reads and rescales
+# them with the vector ALU every tile, and the default AGPR placement costs a copy each way.
+# No NaN reaches these kernels by construction, so fmax needs no operand canonicalisation.
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans"]
+
+
 def _units():
-    units = [("api", "api.hip", []), ("generic", "generic.hip", []), ("dispatch", "dispatch.hip", [])]
+    units = [("api", "api.hip", []), ("generic", "generic.hip", []), ("dispatch", "dispatch.hip", []),
+             ("prep", "prep.hip", [])]
     for d in HEAD_DIMS:
-        units.append((f"mfma_fwd_d{d}", "mfma_fwd.hip", [f"-DEVO_D={d}"]))
-        units.append((f"mfma_bwd_d{d}", "mfma_bwd.hip", [f"-DEVO_D={d}"]))
+        units.append((f"mfma_fwd_d{d}", "mfma_fwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
+        units.append((f"mfma_bwd_d{d}", "mfma_bwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
     return units
 
 

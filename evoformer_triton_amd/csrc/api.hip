@@ -70,6 +70,43 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     *n_chunks = (p.S + *chunk - 1) / *chunk;
 }
 
+struct PrepLayout {
+    size_t bq, bk, m2, dead, total;
+    int bias_batches;
+};
+
+static PrepLayout prep_layout(const EvoAttnParams &p) {
+    PrepLayout w{};
+    const size_t NT = (size_t)(p.N + 31) / 32;
+    w.bias_batches = (p.bias && p.bias_stride_b == 0) ? 1 : p.B;
+    // one extra all-zero tile at the end of each copy
+    const size_t tiles = p.bias ? ((size_t)w.bias_batches * p.H * NT * NT + 1) * 1024 * 4 : 0;
+    size_t off = 0;
+    w.bq = off; off += align_up(tiles);
+    w.bk = off; off += align_up(tiles);
+    w.m2 = off; off += align_up((size_t)p.B * p.S * NT * 32 * 8);
+    w.dead = off; off += align_up((size_t)p.B * p.S * 4);
+    w.total = off;
+    return w;
+}
+
+static void fill_prep(const EvoAttnParams &p, Extra &e) {
+    const PrepLayout w = prep_layout(p);
+    char *base = (char *)p.prep;
+    e.bias_batches = w.bias_batches;
+    e.bq = (float *)(base + w.bq);
+    e.bk = (float *)(base + w.bk);
+    e.m2 = (uint2 *)(base + w.m2);
+    e.dead = (int *)(base + w.dead);
+    e.zero_tile = (int64_t)w.bias_batches * p.H * ((p.N + 31) / 32) * ((p.N + 31) / 32) * 1024;
+}
+
+static int check_prep(const EvoAttnParams &p) {
+    if (!p.prep || p.prep_bytes < prep_layout(p).total) return EVO_EWORKSPACE;
+    if (!aligned(p.prep, 256)) return EVO_EALIGN;
+    return EVO_OK;
+}
+
 struct WsLayout {
     size_t delta, shift, dmask_part, dbias_part, total;
     int n_chunks, chunk;
@@ -133,6 +170,11 @@ int evoattn_check(const EvoAttnParams *p, int pass) {
     return EVO_OK;
 }
 
+size_t evoattn_prep_bytes(const EvoAttnParams *p) {
+    if (!p || p->B <= 0 || p->S <= 0 || p->N <= 0 || p->H <= 0) return 0;
+    return prep_layout(*p).total;
+}
+
 size_t evoattn_bwd_workspace_bytes(const EvoAttnParams *p) {
     if (!p || p->B <= 0 || p->S <= 0 || p->N <= 0 || p->H <= 0) return 0;
     return ws_layout(*p).total;
@@ -148,8 +190,11 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     if (rc) return rc;
     hipStream_t st = (hipStream_t)hip_stream;
     if (!mfma_ok(*p, EVO_PASS_FWD)) return launch_generic_fwd(*p, st);
+    if ((rc = check_prep(*p))) return rc;
     Extra e{};
     e.vec_ok = bias_vec_ok(*p);
+    fill_prep(*p, e);
+    if ((rc = launch_prep(*p, e, st))) return rc;
     return launch_mfma_fwd(*p, e, st);
 }
 
@@ -168,10 +213,12 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     e.dmask_part = (float *)(ws + w.dmask_part);
     e.dbias_part = (float *)(ws + w.dbias_part);
     if (!mfma_ok(*p, EVO_PASS_BWD)) return launch_generic_bwd(*p, e, st);
-    if ((rc = launch_mfma_delta(*p, e, st))) return rc;
-    if ((rc = launch_mask_shift(*p, e, st))) return rc;
-    if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;
+    if ((rc = check_prep(*p))) return rc;
+    fill_prep(*p, e);
+    if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
+    // dQ first: it also writes delta, which the dK/dV kernel reads
     if ((rc = launch_mfma_dq(*p, e, st))) return rc;
+    if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;
     if (p->dbias && (rc = launch_dbias_reduce(*p, e, st))) return rc;
     if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;
     return EVO_OK;

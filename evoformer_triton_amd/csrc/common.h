@@ -26,17 +26,26 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 // A problem whose every key has a mask value below this is shifted by its largest mask
 // value so that the log-sum-exp keeps its mantissa.
-constexpr float kShiftThreshold = -1.0e4f;
+constexpr float kShiftThreshold = -1.0e5f;
+// Most negative additive mask value the matrix-core kernels carry (in log2 units).
+constexpr float kMaskFloor = -1.0e30f;
 
 // Launch-time constants derived on the host.
 struct Extra {
     int n_chunks;      // number of S-chunks the dBias partials are split into
     int chunk;         // rows of S per chunk
     int vec_ok;        // bias rows may be read with 8/16-byte vector loads
+    int bias_batches;  // 1 when one bias is shared by the whole batch, else B
     float *delta;      // [B][H][S][N]
-    float *shift;      // [B][S] per-row mask shift
+    float *shift;      // [B][S] per-row mask shift (plain kernels)
     float *dbias_part; // [n_chunks][B][H][N][N]
     float *dmask_part; // [B][H][S][N]
+    // prepared operands of the matrix-core kernels (written by the prep kernel)
+    float *bq;         // bias * log2(e) in accumulator-tile order, lane = query  [Bb][H][NT][NT][64][16]
+    float *bk;         // same, lane = key
+    uint2 *m2;         // additive mask * log2(e), shifted, clamped, as (hi, mid, lo, 0) of T  [B][S][NT*32]
+    int *dead;         // [B][S] 1 where every key of the row is masked out
+    int64_t zero_tile; // offset (floats) of an all-zero tile inside bq and bk
 };
 
 // Linear block id -> logical id such that consecutive logical ids run on one XCD
@@ -81,6 +90,15 @@ __device__ __forceinline__ float mask_add(const EvoAttnParams &p, int b, int s, 
 }
 
 __device__ __forceinline__ float shift_from_max(float mx) { return mx < kShiftThreshold ? fmaxf(mx, -FLT_MAX) : 0.0f; }
+
+// A bool keep-mask REPLACES the scores of dropped keys (evoformer.py:69, test.py:54), so no
+// gradient reaches Q, K or the bias through them.  Where some key is kept the dropped keys
+// have probability zero and that happens by itself; in a problem whose every key is dropped
+// (shift != 0) the probabilities are uniform and dS has to be cleared explicitly.  dV, which
+// does not pass through the scores, is unaffected.  Additive masks let the gradient through.
+__device__ __forceinline__ bool ds_blocked(const EvoAttnParams &p, float shift) {
+    return p.mask_kind == EVO_MASK_BOOL && shift != 0.0f;
+}
 
 template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 
@@ -134,6 +152,35 @@ __device__ __forceinline__ typename Mfma<T>::v8 zero8() {
 #pragma unroll
     for (int i = 0; i < 8; ++i) z[i] = (T)0.0f;
     return z;
+}
+
+// m = hi + mid + lo with all three representable in T: a fp32 value carried exactly (to
+// 24 bits) through a 16-bit matrix-core operand.  fp16 cannot hold the mask floor; there
+// the value is first clamped to what it can (a score that low has probability zero).
+template <typename T>
+__device__ __forceinline__ void split3(float m, T &hi, T &mid, T &lo) {
+    hi = (T)m;
+    const float r1 = m - (float)hi;
+    mid = (T)r1;
+    lo = (T)(r1 - (float)mid);
+}
+template <>
+__device__ __forceinline__ void split3<f16_t>(float m, f16_t &hi, f16_t &mid, f16_t &lo) {
+    m = fmaxf(m, -60000.0f);
+    hi = (f16_t)m;
+    const float r1 = m - (float)hi;
+    mid = (f16_t)r1;
+    lo = (f16_t)(r1 - (float)mid);
+}
+
+// (hi, mid, lo, 0) of split3 packed into 8 bytes.
+template <typename T>
+__device__ __forceinline__ uint2 pack_split3(float m) {
+    T hi, mid, lo;
+    split3<T>(m, hi, mid, lo);
+    typename Mfma<T>::v4 v;
+    v[0] = hi; v[1] = mid; v[2] = lo; v[3] = (T)0.0f;
+    return __builtin_bit_cast(uint2, v);
 }
 
 // Four bias values for one query row and four consecutive keys, as fp32.

@@ -6,7 +6,6 @@ namespace evo {
 
 #define EVO_DECL(D)                                                                          \
     int launch_mfma_fwd_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
-    int launch_mfma_delta_d##D(const EvoAttnParams &, const Extra &, hipStream_t);           \
     int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
     int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
@@ -26,7 +25,6 @@ EVO_DECL(64)
         return EVO_EUNSUPPORTED;                                              \
     }
 EVO_ROUTE(fwd)
-EVO_ROUTE(delta)
 EVO_ROUTE(dq)
 EVO_ROUTE(dkdv)
 #undef EVO_ROUTE

@@ -88,6 +88,7 @@ __global__ void __launch_bounds__(64) gen_dq(EvoAttnParams p, const float *delta
     load_row(G + (int64_t)rowc * p.stride_n, g, D);
     for (int d = 0; d < D; ++d) acc[d] = 0.0f;
     const float shift = shift_tab[pr.b * p.S + pr.s];
+    const bool kill = ds_blocked(p, shift);
     const float lse = p.lse[pr.row0 + rowc], dl = delta[pr.row0 + rowc];
     const int64_t brow = (int64_t)pr.b * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h + (int64_t)rowc * p.bias_stride_row;
     for (int j = 0; j < p.N; ++j) {
@@ -98,7 +99,7 @@ __global__ void __launch_bounds__(64) gen_dq(EvoAttnParams p, const float *delta
             dp = fmaf(g[d], (float)vr[d], dp);
         }
         float t = score<BIASK, T>(p, qk, brow + j, mask_add(p, pr.b, pr.s, j), shift);
-        float ds = expf(t - lse) * (dp - dl);
+        float ds = kill ? 0.0f : expf(t - lse) * (dp - dl);
         for (int d = 0; d < D; ++d) acc[d] = fmaf(ds, (float)kr[d], acc[d]);
     }
     if (row < p.N) {
@@ -121,6 +122,7 @@ __global__ void __launch_bounds__(64) gen_dkdv(EvoAttnParams p, const float *del
     load_row(V + (int64_t)keyc * p.stride_n, v, D);
     for (int d = 0; d < D; ++d) dk[d] = dv[d] = 0.0f;
     const float shift = shift_tab[pr.b * p.S + pr.s];
+    const bool kill = ds_blocked(p, shift);
     const float mk = mask_add(p, pr.b, pr.s, keyc);
     const int64_t bcol = (int64_t)pr.b * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h + keyc;
     float dm = 0.0f;
@@ -133,7 +135,7 @@ __global__ void __launch_bounds__(64) gen_dkdv(EvoAttnParams p, const float *del
         }
         float t = score<BIASK, T>(p, qk, bcol + (int64_t)i * p.bias_stride_row, mk, shift);
         float pij = expf(t - p.lse[pr.row0 + i]);
-        float ds = pij * (dp - delta[pr.row0 + i]);
+        float ds = kill ? 0.0f : pij * (dp - delta[pr.row0 + i]);
         for (int d = 0; d < D; ++d) {
             dv[d] = fmaf(pij, (float)gr[d], dv[d]);
             dk[d] = fmaf(ds, (float)qr[d], dk[d]);
@@ -181,7 +183,9 @@ __global__ void __launch_bounds__(64) gen_dbias(EvoAttnParams p, const float *de
             qk = fmaf((float)qr[d], (float)kr[d], qk);
             dp = fmaf((float)gr[d], (float)vr[d], dp);
         }
-        float t = score<BIASK, T>(p, qk, boff, mask_add(p, b, s, j), shift_tab[b * p.S + s]);
+        const float shift = shift_tab[b * p.S + s];
+        if (ds_blocked(p, shift)) continue;
+        float t = score<BIASK, T>(p, qk, boff, mask_add(p, b, s, j), shift);
         acc += expf(t - p.lse[pr.row0 + i]) * (dp - delta[pr.row0 + i]);
     }
     store_typed(p.dbias, p.dbias_dtype, (((int64_t)b * p.H + h) * p.N + i) * p.N + j, acc);

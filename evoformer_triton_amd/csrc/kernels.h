@@ -13,8 +13,8 @@ int launch_dmask_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_dbias_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mask_shift(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 
+int launch_prep(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_fwd(const EvoAttnParams &p, const Extra &e, hipStream_t st);
-int launch_mfma_delta(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_dkdv(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 

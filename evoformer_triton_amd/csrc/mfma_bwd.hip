@@ -2,18 +2,26 @@
 // Compiled once per head dim (-DEVO_D=8|16|32|64).
 //
 // They replace the reference's `_attn_bwd_preprocess` (evoformer.py:299-326),
-// `_attn_bwd_dq` (:329-476) and `_attn_bwd_dk_dv` (:479-630).  Both big kernels recompute
+// `_attn_bwd_dq` (:329-476) and `_attn_bwd_dk_dv` (:479-630).  Both kernels recompute
 // P = exp(score - LSE) from the saved log-sum-exp (:452, :600), form
 // dS = P * (dP - delta) (:456, :610) and cast P and dS to the input dtype before the
 // gradient matmuls (:459, :603, :611); dQ and dK are multiplied by the softmax scale after
 // the matmul (:462, :614).
 //
+// As in the forward, the vector ALU is the scarce unit (one exp per score, twice), so every
+// addition is folded into the matrix core: one operand is pre-multiplied by
+// scale*log2(e), the bias tile (log2 units, accumulator order, see prep.hip) is the C
+// operand of the score MFMA, and mask, -LSE and -delta travel as three 16-bit columns
+// each (hi + mid + lo, exact to 24 bits) in one extra k-step against columns of ones.
+// The score MFMA then yields log2 P directly and the dO.V^T MFMA yields dP - delta; per
+// score there remain exp2, one multiply and the two conversions.
+//
 // dBias is the sum of dS over S.  The reference adds every fp32 dS tile into global memory
 // with atomics (:458).  Here the dQ kernel owns a 32-query slab of one head for a whole
 // chunk of S rows and keeps the running sum of dS for that slab in matrix-core
-// accumulators (an identity-matrix MFMA adds the bf16 dS tile that the dQ matmul consumes
-// anyway), writes one partial per chunk, and a second kernel adds the partials in a fixed
-// order: no floating-point atomics, bit-reproducible.
+// accumulators (an identity-matrix MFMA adds the dS tile, rounded to fp16 for this purpose:
+// 11 significant bits per term, fp32 sum), writes one partial per chunk, and a second
+// kernel adds the partials in a fixed order: no floating-point atomics, bit-reproducible.
 #include "common.h"
 #include "kernels.h"
 
@@ -23,48 +31,72 @@
 
 namespace evo {
 
-// delta[row] = sum_d dO[row,d] * O[row,d]  (evoformer.py:313-323)
-template <typename T, int D>
-__global__ void __launch_bounds__(256) mfma_delta(EvoAttnParams p, float *delta) {
-    typedef typename Mfma<T>::v8 v8;
-    const int64_t rows = (int64_t)p.B * p.H * p.S * p.N;
-    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (r >= rows) return;
-    const Prob pr = decode_problem(p, (unsigned)(r / p.N));
-    const int64_t off = pr.base + (r % p.N) * p.stride_n;
-    const T *O = (const T *)p.o + off, *G = (const T *)p.dout + off;
-    float s = 0.0f;
+// Geometry shared by the two kernels for head dim D.
+template <int D>
+struct Geo {
+    static constexpr bool AUG_IN_PAD = D == 8;           // extra columns fit the zero padding of k-step 0
+    static constexpr int KW = AUG_IN_PAD ? 16 : D + 16;  // operand row: data, extra columns, zeros
+    static constexpr int KS = KW / 16;
+    static constexpr int KSD = (D + 15) / 16;            // k-steps that hold data
+    static constexpr int AUGC = AUG_IN_PAD ? 8 : D;      // first extra column
+    static constexpr int DT = (D + 31) / 32;
+    static constexpr int DP = DT * 32;
+};
+
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 scaled8(typename Mfma<T>::v8 raw, float c) {
+    typename Mfma<T>::v8 r;
 #pragma unroll
-    for (int c = 0; c < D / 8; ++c) {
-        v8 o = ld8(O + c * 8), g = ld8(G + c * 8);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) s = fmaf((float)g[i], (float)o[i], s);
-    }
-    delta[r] = s;
+    for (int i = 0; i < 8; ++i) r[i] = (T)((float)raw[i] * c);
+    return r;
 }
 
-// ------------------------------------------------------------------ dQ and dBias partials
+// 8 operand columns [a0 a1 a2 b0 b1 b2 0 0] from two packed (hi, mid, lo, 0) triples.
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 aug8(uint2 a, uint2 b) {
+    typename Mfma<T>::v4 va = __builtin_bit_cast(typename Mfma<T>::v4, a);
+    typename Mfma<T>::v4 vb = __builtin_bit_cast(typename Mfma<T>::v4, b);
+    typename Mfma<T>::v8 r;
+    r[0] = va[0]; r[1] = va[1]; r[2] = va[2];
+    r[3] = vb[0]; r[4] = vb[1]; r[5] = vb[2];
+    r[6] = (T)0.0f; r[7] = (T)0.0f;
+    return r;
+}
+
+template <typename T>
+__device__ __forceinline__ uint2 ones3() {
+    typename Mfma<T>::v4 v;
+    v[0] = v[1] = v[2] = (T)1.0f;
+    v[3] = (T)0.0f;
+    return __builtin_bit_cast(uint2, v);
+}
+
+// ------------------------------------------------------------------ dQ, delta and dBias partials
 //
 // Workgroup = 4 waves = (b, h, chunk of S, 32 query rows).  The waves split the keys:
 // wave w takes 32-key tiles w, w+4, w+8, ...  Scores are computed transposed
 // (S^T = K Q^T, dP^T = V dO^T) so that a lane owns one query and 16 keys, which makes the
 // dS^T accumulator tile the B operand of both dQ^T += K^T dS^T and dBias^T += I dS^T.
 // Each wave's partial dQ^T meets the others in LDS once per S row and is summed in wave
-// order.
-template <typename T, int D, int BIASK, int NTW>
+// order.  Query slab and head are fixed for the whole S loop, so for N <= 512 the bias
+// tiles stay in registers across it.  delta = rowsum(dO * O) (evoformer.py:313-323) is
+// formed here from the rows the kernel loads anyway and written out for the dK/dV kernel.
+template <typename T, int D, bool HAS_BIAS, int NTW>
 __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
-    constexpr int DK = D < 16 ? 16 : D;
-    constexpr int KS = DK / 16;
-    constexpr int DT = (D + 31) / 32;
-    constexpr int RP = DT * 32 + 4;  // pitch of a partial dQ row in LDS (floats)
+    typedef Geo<D> G;
+    constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
+    constexpr int RP = DT * 32 + 4;   // pitch of a partial dQ row in LDS (floats)
+    constexpr int KTP = 32 + 8;       // pitch of a transposed K tile row
+    constexpr bool BIAS_RESIDENT = HAS_BIAS && NTW <= 4;
+    constexpr int NRES = BIAS_RESIDENT ? NTW : 1;
     typedef typename Mfma<T>::v8 v8;
 
-    __shared__ __attribute__((aligned(16))) float Ms[NTW * 128];
     __shared__ __attribute__((aligned(16))) float red[4 * 32 * RP];
+    __shared__ __attribute__((aligned(16))) T Kt[4 * DP * KTP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
-    const int NT = (p.N + 31) / 32;
+    const int NT = (p.N + 31) / 32, npad = NT * 32;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const int qt = lid % NT;
     const unsigned bh = (lid / NT) % (unsigned)(p.B * p.H);
@@ -73,18 +105,21 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
     const int q0 = qt * 32;
     const int qrow = min(q0 + li, p.N - 1);
     const int64_t sn = p.stride_n;
-    const int64_t brow = (int64_t)b * p.bias_stride_b + (int64_t)h * p.bias_stride_h + (int64_t)qrow * p.bias_stride_row;
-    const bool vec = e.vec_ok != 0;
     const bool want_dbias = e.dbias_part != nullptr && p.dbias != nullptr;
-    const float scale = p.scale;
+    const float cs = p.scale * kLog2e;
+    T *Ktw = Kt + wave * DP * KTP;
 
-    // identity slices: A[m][8g+i] = 1 where m is the key row that register 8ts+i of a
-    // C-layout tile holds for lane group g
-    v8 idf[2];
+    // rows d >= D of the transposed K tile are read by the MFMA but never written
+    if (DP > D)
+        for (int i = lane; i < (DP - D) * KTP; i += 64) Ktw[D * KTP + i] = (T)0.0f;
+
+    // identity slices in fp16: A[m][8g+i] = 1 where m is the key row that register 8ts+i of
+    // an accumulator tile holds for lane group g
+    f16x8 idf[2];
 #pragma unroll
     for (int ts = 0; ts < 2; ++ts)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) idf[ts][i] = (T)(li == crow(8 * ts + i, g) ? 1.0f : 0.0f);
+        for (int i = 0; i < 8; ++i) idf[ts][i] = (f16_t)(li == crow(8 * ts + i, g) ? 1.0f : 0.0f);
 
     f32x16 dbacc[NTW];
 #pragma unroll
@@ -92,25 +127,61 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
 
+    const int bb = e.bias_batches > 1 ? b : 0;
+    const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
+    const float *ztile = e.bq + e.zero_tile + lane * 16;
+    auto load_btile = [&](const float *src, f32x16 &dst) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
+            dst[4 * rr] = v[0]; dst[4 * rr + 1] = v[1]; dst[4 * rr + 2] = v[2]; dst[4 * rr + 3] = v[3];
+        }
+    };
+    f32x16 bres[NRES];
+    if (BIAS_RESIDENT) {
+#pragma unroll
+        for (int j = 0; j < NRES; ++j) load_btile(btile0 + (int64_t)min(wave + 4 * j, NT - 1) * 1024, bres[j]);
+    }
+
+    const uint2 one3 = ones3<T>();
+    const uint2 zero3 = {0u, 0u};
     const int s_begin = c * e.chunk, s_end = min(p.S, s_begin + e.chunk);
     for (int s = s_begin; s < s_end; ++s) {
         const unsigned pid = (bh * (unsigned)p.S) + s;
         const Prob pr = decode_problem(p, pid);
         const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
-        const T *G = (const T *)p.dout + pr.base;
+        const T *Gd = (const T *)p.dout + pr.base, *O = (const T *)p.o + pr.base;
+        const uint2 *m2row = e.m2 + ((int64_t)b * p.S + s) * npad;
+        const bool dead = e.dead[b * p.S + s] != 0;
+        const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
 
-        __syncthreads();  // last row's readers of Ms and red are done
-        for (int j = tid; j < NTW * 128; j += 256) Ms[j] = mask_add(p, b, s, j);
-        const float shift = e.shift[b * p.S + s];
+        // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
         v8 qf[KS], gf[KS];
+        float dpart = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int d0 = ks * 16 + g * 8;
-            qf[ks] = d0 < D ? ld8(Q + (int64_t)qrow * sn + d0) : zero8<T>();
-            gf[ks] = d0 < D ? ld8(G + (int64_t)qrow * sn + d0) : zero8<T>();
+            qf[ks] = zero8<T>();
+            gf[ks] = zero8<T>();
+            if (d0 < D) {
+                v8 qraw = ld8(Q + (int64_t)qrow * sn + d0);
+                gf[ks] = ld8(Gd + (int64_t)qrow * sn + d0);
+                v8 oraw = ld8(O + (int64_t)qrow * sn + d0);
+                if (!dead) qf[ks] = scaled8<T>(qraw, cs);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) dpart = fmaf((float)gf[ks][i], (float)oraw[i], dpart);
+            }
         }
-        const float lse = p.lse[pr.row0 + qrow], dl = e.delta[pr.row0 + qrow];
-        __syncthreads();
+        const float dl = dpart + __shfl_xor(dpart, 32);
+        const float lse2 = p.lse[pr.row0 + qrow] * kLog2e;
+        if (wave == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks * 16 + g * 8 == AUGC) {
+                qf[ks] = aug8<T>(one3, pack_split3<T>(-lse2));   // ones x mask, -lse x ones
+                gf[ks] = aug8<T>(pack_split3<T>(-dl), zero3);    // -delta x ones
+            }
+        }
 
         f32x16 dqacc[DT];
 #pragma unroll
@@ -121,60 +192,87 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 #pragma unroll 1
         for (int j = 0; j < NTW; ++j) {
             const int kt = wave + 4 * j;
-            if (kt * 32 < p.N) {  // wave-uniform
+            if (kt < NT) {  // wave-uniform
                 const int kb = kt * 32;
                 const int keyc = min(kb + li, p.N - 1);
-                f32x16 acc, dp;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = dp[r] = 0.0f;
+                v8 ka[KS], va[KS];
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     const int d0 = ks * 16 + g * 8;
-                    v8 ka = d0 < D ? ld8(K + (int64_t)keyc * sn + d0) : zero8<T>();
-                    v8 va = d0 < D ? ld8(V + (int64_t)keyc * sn + d0) : zero8<T>();
-                    acc = Mfma<T>::mma(ka, qf[ks], acc);
-                    dp = Mfma<T>::mma(va, gf[ks], dp);
+                    ka[ks] = zero8<T>();
+                    va[ks] = zero8<T>();
+                    if (d0 < D) {
+                        ka[ks] = ld8(K + (int64_t)keyc * sn + d0);
+                        va[ks] = ld8(V + (int64_t)keyc * sn + d0);
+                    } else if (d0 == AUGC) {
+                        ka[ks] = aug8<T>(m2row[kb + li], one3);  // mask x ones, ones x -lse
+                        va[ks] = aug8<T>(one3, zero3);           // ones x -delta
+                    }
+                }
+                // transposed copy of the K tile for dQ^T += K^T dS^T (wave-private LDS)
+#pragma unroll
+                for (int ks = 0; ks < KSD; ++ks) {
+                    const int d0 = ks * 16 + g * 8;
+                    if (d0 < D) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) Ktw[(d0 + i) * KTP + perm_pos(li)] = ka[ks][i];
+                    }
+                }
+                f32x16 acc, dp;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = dp[r] = 0.0f;
+                if (HAS_BIAS) {
+                    if (BIAS_RESIDENT) {
+                        // compare chain: a static register index for a run-time tile number
+#pragma unroll
+                        for (int jj = 0; jj < NRES; ++jj)
+                            if (jj == j) acc = bres[jj];
+                        if (dead) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+                        }
+                    } else {
+                        load_btile(dead ? ztile : btile0 + (int64_t)kt * 1024, acc);
+                    }
+                }
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    acc = Mfma<T>::mma(ka[ks], qf[ks], acc);   // log2 P^T
+                    dp = Mfma<T>::mma(va[ks], gf[ks], dp);     // dP^T - delta
                 }
                 float ds[16];
 #pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int kg = kb + 8 * rr + 4 * g;
-                    float bv[4];
-                    load_bias4<BIASK, T>(p.bias, brow + kg, p.N - kg, vec, bv);
-                    const f32x4 mk = *reinterpret_cast<const f32x4 *>(&Ms[kg]);
+                for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(acc[r]) * dp[r];
+                if (kill) {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        float t = fmaf(acc[4 * rr + i], scale, bv[i]) + mk[i];
-                        if (shift != 0.0f) t -= shift;
-                        const float pv = fast_exp2((t - lse) * kLog2e);
-                        ds[4 * rr + i] = pv * (dp[4 * rr + i] - dl);
-                    }
+                    for (int r = 0; r < 16; ++r) ds[r] = 0.0f;
                 }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
                 for (int ts = 0; ts < 2; ++ts) {
                     v8 dsf;
+                    f16x8 dsh;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) dsf[i] = (T)ds[8 * ts + i];
+                    for (int i = 0; i < 8; ++i) {
+                        dsf[i] = (T)ds[8 * ts + i];
+                        dsh[i] = (f16_t)ds[8 * ts + i];
+                    }
                     if (want_dbias) {
-                        // j is a run-time value here; the compare chain keeps the
-                        // accumulator index static so the tiles stay in registers
 #pragma unroll
                         for (int jj = 0; jj < NTW; ++jj)
-                            if (jj == j) dbacc[jj] = Mfma<T>::mma(idf[ts], dsf, dbacc[jj]);
+                            if (jj == j) dbacc[jj] = Mfma<f16_t>::mma(idf[ts], dsh, dbacc[jj]);
                     }
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
-                        // K^T operand: row d, columns = the keys registers 8ts..8ts+7 hold
-                        const int d = dt * 32 + li;
-                        v8 kta;
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) {
-                            const int key = min(kb + crow(8 * ts + i, g), p.N - 1);
-                            kta[i] = d < D ? K[(int64_t)key * sn + d] : (T)0.0f;
-                        }
+                        v8 kta = *reinterpret_cast<const v8 *>(&Ktw[(dt * 32 + li) * KTP + ts * 16 + g * 8]);
                         dqacc[dt] = Mfma<T>::mma(kta, dsf, dqacc[dt]);
                     }
                 }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
         }
 
@@ -196,8 +294,10 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 #pragma unroll
             for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[(w * 32 + q) * RP + d4]);
             if (q0 + q < p.N)
-                store4<T>(dQ + (int64_t)(q0 + q) * sn + d4, sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
+                store4<T>(dQ + (int64_t)(q0 + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
+                          sum[3] * p.scale);
         }
+        __syncthreads();  // red is rewritten by the next S row
     }
 
     if (want_dbias && q0 + li < p.N) {
@@ -229,18 +329,18 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 // ------------------------------------------------------------------ dK, dV (and dMask partials)
 //
 // Workgroup = 4 waves = 128 keys of one problem; each wave keeps its 32 keys' K and V
-// operands in registers and loops over all query rows, staged 64 at a time through LDS both
-// row-major (for S = Q K^T, dP = dO V^T) and transposed (for dV^T += dO^T P, dK^T += Q^T dS).
+// operands in registers and loops over all query rows, staged through LDS both row-major
+// (for S = Q K^T, dP = dO V^T) and transposed (for dV^T += dO^T P, dK^T += Q^T dS).
 // Scores are NOT transposed here: a lane owns one key and 16 queries, so that P and dS in
 // accumulator layout are the B operands of the two gradient matmuls.
-template <typename T, int D, int BIASK>
+template <typename T, int D, bool HAS_BIAS>
 __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
-    constexpr int BK = 128, BQS = 64;
-    constexpr int DK = D < 16 ? 16 : D;
-    constexpr int KS = DK / 16;
-    constexpr int DT = (D + 31) / 32;
-    constexpr int DP = DT * 32;
-    constexpr int QP = DK + 8;
+    typedef Geo<D> G;
+    constexpr int KW = G::KW, KS = G::KS, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
+    constexpr int BK = 128;
+    constexpr int BQS = D <= 32 ? 128 : 64;  // query rows staged per round
+    constexpr int TPS = BQS / 32;            // query tiles per stage
+    constexpr int QP = KW + 8;
     constexpr int TP = BQS + 8;
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v2 v2;
@@ -249,37 +349,71 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
     __shared__ __attribute__((aligned(16))) T Gs[BQS * QP];
     __shared__ __attribute__((aligned(16))) T Qt[DP * TP];
     __shared__ __attribute__((aligned(16))) T Gt[DP * TP];
-    __shared__ __attribute__((aligned(16))) float Ls[BQS];
-    __shared__ __attribute__((aligned(16))) float Ds[BQS];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
+    const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nkb = (p.N + BK - 1) / BK;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nkb;
     const int key0 = (lid % nkb) * BK + wave * 32;
     const Prob pr = decode_problem(p, pid);
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
-    const T *G = (const T *)p.dout + pr.base;
+    const T *Gd = (const T *)p.dout + pr.base;
     const int64_t sn = p.stride_n;
     const bool active = key0 < p.N;
     const int key = key0 + li, keyc = min(key, p.N - 1);
-    const float scale = p.scale;
+    const bool dead = e.dead[pr.b * p.S + pr.s] != 0;
+    const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
+    const bool want_dm = e.dmask_part != nullptr && p.dmask != nullptr;
+    const float cs = p.scale * kLog2e;
+    const uint2 one3 = ones3<T>();
+    const uint2 zero3 = {0u, 0u};
 
-    for (int i = tid; i < BQS * QP; i += 256) Qs[i] = Gs[i] = (T)0.0f;
-    for (int i = tid; i < DP * TP; i += 256) Qt[i] = Gt[i] = (T)0.0f;
+    // LDS that is read but never staged
+    if (!G::AUG_IN_PAD)
+        for (int r = tid; r < BQS; r += 256) {
+            *reinterpret_cast<v8 *>(&Qs[r * QP + AUGC + 8]) = zero8<T>();
+            *reinterpret_cast<v8 *>(&Gs[r * QP + AUGC + 8]) = zero8<T>();
+        }
+    if (DP > D)
+        for (int i = tid; i < (DP - D) * TP / 8; i += 256) {
+            *reinterpret_cast<v8 *>(&Qt[D * TP + i * 8]) = zero8<T>();
+            *reinterpret_cast<v8 *>(&Gt[D * TP + i * 8]) = zero8<T>();
+        }
 
+    // this wave's keys: K with the mask columns, V with ones against -delta
     v8 kf[KS], vf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 16 + g * 8;
-        kf[ks] = d0 < D ? ld8(K + (int64_t)keyc * sn + d0) : zero8<T>();
-        vf[ks] = d0 < D ? ld8(V + (int64_t)keyc * sn + d0) : zero8<T>();
+        kf[ks] = zero8<T>();
+        vf[ks] = zero8<T>();
+        if (d0 < D) {
+            if (!dead) kf[ks] = ld8(K + (int64_t)keyc * sn + d0);
+            vf[ks] = ld8(V + (int64_t)keyc * sn + d0);
+        } else if (d0 == AUGC) {
+            const int kk = min(key, npad - 1);
+            kf[ks] = aug8<T>(e.m2[((int64_t)pr.b * p.S + pr.s) * npad + kk], one3);  // mask x ones, ones x -lse
+            vf[ks] = aug8<T>(one3, zero3);                                           // ones x -delta
+        }
     }
-    const float mk = mask_add(p, pr.b, pr.s, key);
-    const float shift = e.shift[pr.b * p.S + pr.s];
-    const int64_t bcol = (int64_t)pr.b * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h + keyc;
-    const bool want_dm = e.dmask_part != nullptr && p.dmask != nullptr;
+
+    const int bb = e.bias_batches > 1 ? pr.b : 0;
+    const int ktc = min(key0 >> 5, NT - 1);
+    const float *btile = dead ? e.bk + e.zero_tile + lane * 16
+                              : e.bk + (((int64_t)bb * p.H + pr.h) * NT * NT + ktc) * 1024 + lane * 16;
+    const int64_t bstep = dead ? 0 : (int64_t)NT * 1024;  // next query tile, same key tile
+    auto load_btile = [&](int qt, f32x16 &dst) {
+        if (HAS_BIAS) {
+            const float *src = btile + (int64_t)min(qt, NT - 1) * bstep;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
+                dst[4 * rr] = v[0]; dst[4 * rr + 1] = v[1]; dst[4 * rr + 2] = v[2]; dst[4 * rr + 3] = v[3];
+            }
+        }
+    };
 
     f32x16 dk[DT], dv[DT];
 #pragma unroll
@@ -288,90 +422,110 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
         for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.0f;
     float dm = 0.0f;
 
-    for (int qs0 = 0; qs0 < p.N; qs0 += BQS) {
+    auto stage = [&](int qs0) {
         __syncthreads();
         for (int it = tid; it < BQS * (D / 8); it += 256) {
-            const int row = it / (D / 8), c = it % (D / 8), qq = qs0 + row;
-            v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + c * 8) : zero8<T>();
-            v8 bb = qq < p.N ? ld8(G + (int64_t)qq * sn + c * 8) : zero8<T>();
-            *reinterpret_cast<v8 *>(&Qs[row * QP + c * 8]) = a;
-            *reinterpret_cast<v8 *>(&Gs[row * QP + c * 8]) = bb;
+            const int row = it / (D / 8), ch = it % (D / 8), qq = qs0 + row;
+            v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + ch * 8) : zero8<T>();
+            v8 bb2 = qq < p.N ? ld8(Gd + (int64_t)qq * sn + ch * 8) : zero8<T>();
+            // the score operand carries scale*log2(e), rounded exactly as in the forward
+            *reinterpret_cast<v8 *>(&Qs[row * QP + ch * 8]) = scaled8<T>(a, cs);
+            *reinterpret_cast<v8 *>(&Gs[row * QP + ch * 8]) = bb2;
         }
-        for (int it = tid; it < (BQS / 2) * (D / 8); it += 256) {
-            const int jp = it / (D / 8), c = it % (D / 8), r0 = qs0 + 2 * jp;
-            v8 qa = r0 < p.N ? ld8(Q + (int64_t)r0 * sn + c * 8) : zero8<T>();
-            v8 qb = r0 + 1 < p.N ? ld8(Q + (int64_t)(r0 + 1) * sn + c * 8) : zero8<T>();
-            v8 ga = r0 < p.N ? ld8(G + (int64_t)r0 * sn + c * 8) : zero8<T>();
-            v8 gb = r0 + 1 < p.N ? ld8(G + (int64_t)(r0 + 1) * sn + c * 8) : zero8<T>();
+        for (int row = tid; row < BQS; row += 256) {
+            const int qq = qs0 + row;
+            // rows past N get -LSE = floor: their probabilities vanish
+            const float nl = qq < p.N ? -p.lse[pr.row0 + qq] * kLog2e : kMaskFloor;
+            const float nd = qq < p.N ? -e.delta[pr.row0 + qq] : 0.0f;
+            *reinterpret_cast<v8 *>(&Qs[row * QP + AUGC]) = aug8<T>(one3, pack_split3<T>(nl));
+            *reinterpret_cast<v8 *>(&Gs[row * QP + AUGC]) = aug8<T>(pack_split3<T>(nd), zero3);
+        }
+        constexpr int NPAIR = BQS / 2;
+        for (int it = tid; it < NPAIR * (D / 8); it += 256) {
+            const int ch = it / NPAIR, jp = it % NPAIR, r0 = qs0 + 2 * jp;
+            v8 qa = r0 < p.N ? ld8(Q + (int64_t)r0 * sn + ch * 8) : zero8<T>();
+            v8 qb = r0 + 1 < p.N ? ld8(Q + (int64_t)(r0 + 1) * sn + ch * 8) : zero8<T>();
+            v8 ga = r0 < p.N ? ld8(Gd + (int64_t)r0 * sn + ch * 8) : zero8<T>();
+            v8 gb = r0 + 1 < p.N ? ld8(Gd + (int64_t)(r0 + 1) * sn + ch * 8) : zero8<T>();
             const int pos = perm_pos(2 * jp);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 v2 w;
                 w[0] = qa[i]; w[1] = qb[i];
-                *reinterpret_cast<v2 *>(&Qt[(c * 8 + i) * TP + pos]) = w;
+                *reinterpret_cast<v2 *>(&Qt[(ch * 8 + i) * TP + pos]) = w;
                 w[0] = ga[i]; w[1] = gb[i];
-                *reinterpret_cast<v2 *>(&Gt[(c * 8 + i) * TP + pos]) = w;
+                *reinterpret_cast<v2 *>(&Gt[(ch * 8 + i) * TP + pos]) = w;
             }
-        }
-        if (tid < BQS) {
-            const int qq = qs0 + tid;
-            Ls[tid] = qq < p.N ? p.lse[pr.row0 + qq] : INFINITY;
-            Ds[tid] = qq < p.N ? e.delta[pr.row0 + qq] : 0.0f;
         }
         __syncthreads();
+    };
 
-        if (active) {
+    // one 32-query tile against this wave's 32 keys
+    auto compute = [&](int qtile, const f32x16 &ctile) {
+        const int qb = (qtile % TPS) * 32;
+        f32x16 acc, dp;
 #pragma unroll
-            for (int qt = 0; qt < BQS / 32; ++qt) {
-                const int qb = qt * 32;
-                if (qs0 + qb >= p.N) break;
-                f32x16 acc, dp;
+        for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = dp[r] = 0.0f;
+        for (int ks = 0; ks < KS; ++ks) {
+            v8 qa = *reinterpret_cast<const v8 *>(&Qs[(qb + li) * QP + ks * 16 + g * 8]);
+            v8 ga = *reinterpret_cast<const v8 *>(&Gs[(qb + li) * QP + ks * 16 + g * 8]);
+            if (ks == 0) {
+                if (HAS_BIAS) {
+                    acc = Mfma<T>::mma(qa, kf[0], ctile);
+                } else {
+                    f32x16 z;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    v8 qa = *reinterpret_cast<const v8 *>(&Qs[(qb + li) * QP + ks * 16 + g * 8]);
-                    v8 ga = *reinterpret_cast<const v8 *>(&Gs[(qb + li) * QP + ks * 16 + g * 8]);
-                    acc = Mfma<T>::mma(qa, kf[ks], acc);
-                    dp = Mfma<T>::mma(ga, vf[ks], dp);
+                    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                    acc = Mfma<T>::mma(qa, kf[0], z);
                 }
-                float pv[16], ds[16];
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int ql = qb + 8 * rr + 4 * g;
-                    const f32x4 l4 = *reinterpret_cast<const f32x4 *>(&Ls[ql]);
-                    const f32x4 d4 = *reinterpret_cast<const f32x4 *>(&Ds[ql]);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int qg = min(qs0 + ql + i, p.N - 1);
-                        const float bv = load_bias1<BIASK, T>(p.bias, bcol + (int64_t)qg * p.bias_stride_row);
-                        float t = fmaf(acc[4 * rr + i], scale, bv) + mk;
-                        if (shift != 0.0f) t -= shift;
-                        pv[4 * rr + i] = fast_exp2((t - l4[i]) * kLog2e);
-                        ds[4 * rr + i] = pv[4 * rr + i] * (dp[4 * rr + i] - d4[i]);
-                    }
-                }
-                if (want_dm) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) dm += ds[r];
-                }
-#pragma unroll
-                for (int ts = 0; ts < 2; ++ts) {
-                    v8 pf, dsf;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        pf[i] = (T)pv[8 * ts + i];
-                        dsf[i] = (T)ds[8 * ts + i];
-                    }
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        v8 ga = *reinterpret_cast<const v8 *>(&Gt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
-                        v8 qa = *reinterpret_cast<const v8 *>(&Qt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
-                        dv[dt] = Mfma<T>::mma(ga, pf, dv[dt]);
-                        dk[dt] = Mfma<T>::mma(qa, dsf, dk[dt]);
-                    }
-                }
+            } else {
+                acc = Mfma<T>::mma(qa, kf[ks], acc);           // log2 P
             }
+            dp = Mfma<T>::mma(ga, vf[ks], dp);                 // dP - delta
+        }
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            acc[r] = fast_exp2(acc[r]);
+            ds[r] = acc[r] * dp[r];
+        }
+        if (kill) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = 0.0f;
+        }
+        if (want_dm) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dm += ds[r];
+        }
+#pragma unroll
+        for (int ts = 0; ts < 2; ++ts) {
+            v8 pf, dsf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pf[i] = (T)acc[8 * ts + i];
+                dsf[i] = (T)ds[8 * ts + i];
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                v8 ga = *reinterpret_cast<const v8 *>(&Gt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
+                v8 qa = *reinterpret_cast<const v8 *>(&Qt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
+                dv[dt] = Mfma<T>::mma(ga, pf, dv[dt]);
+                dk[dt] = Mfma<T>::mma(qa, dsf, dk[dt]);
+            }
+        }
+    };
+
+    // query tiles in pairs on two register sets (bias tile of the next one in flight)
+    f32x16 tA, tB;
+    load_btile(0, tA);
+    for (int qtile = 0; qtile < NT; qtile += 2) {
+        if (qtile % TPS == 0) stage(qtile * 32);
+        load_btile(qtile + 1, tB);
+        if (active) compute(qtile, tA);
+        if (qtile + 1 < NT) {
+            load_btile(qtile + 2, tA);
+            if (active) compute(qtile + 1, tB);
         }
     }
 
@@ -389,8 +543,8 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
                 for (int rr = 0; rr < 4; ++rr) {
                     const int d0 = dt * 32 + 8 * rr + 4 * g;
                     if (d0 < D) {
-                        store4<T>(dK + d0, dk[dt][4 * rr] * scale, dk[dt][4 * rr + 1] * scale,
-                                  dk[dt][4 * rr + 2] * scale, dk[dt][4 * rr + 3] * scale);
+                        store4<T>(dK + d0, dk[dt][4 * rr] * p.scale, dk[dt][4 * rr + 1] * p.scale,
+                                  dk[dt][4 * rr + 2] * p.scale, dk[dt][4 * rr + 3] * p.scale);
                         store4<T>(dV + d0, dv[dt][4 * rr], dv[dt][4 * rr + 1], dv[dt][4 * rr + 2], dv[dt][4 * rr + 3]);
                     }
                 }
@@ -405,40 +559,29 @@ static inline int hip_rc() {
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }
 
-template <typename T, int D, int BIASK>
+template <typename T, int D, bool HAS_BIAS>
 static int dq_ntw(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const int NT = (p.N + 31) / 32;
     const unsigned grid = (unsigned)NT * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
     const int ntw = (NT + 3) / 4;
-    if (ntw <= 2) mfma_dq<T, D, BIASK, 2><<<grid, 256, 0, st>>>(p, e);
-    else if (ntw <= 4) mfma_dq<T, D, BIASK, 4><<<grid, 256, 0, st>>>(p, e);
-    else if (ntw <= 8) mfma_dq<T, D, BIASK, 8><<<grid, 256, 0, st>>>(p, e);
-    else if (ntw <= 16) mfma_dq<T, D, BIASK, 16><<<grid, 256, 0, st>>>(p, e);
+    if (ntw <= 2) mfma_dq<T, D, HAS_BIAS, 2><<<grid, 256, 0, st>>>(p, e);
+    else if (ntw <= 4) mfma_dq<T, D, HAS_BIAS, 4><<<grid, 256, 0, st>>>(p, e);
+    else if (ntw <= 8) mfma_dq<T, D, HAS_BIAS, 8><<<grid, 256, 0, st>>>(p, e);
+    else if (ntw <= 16) mfma_dq<T, D, HAS_BIAS, 16><<<grid, 256, 0, st>>>(p, e);
     else return EVO_EUNSUPPORTED;
     return hip_rc();
 }
 
 template <typename T, int D>
 static int dq_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    if (p.bias_dtype == EVO_NONE) return dq_ntw<T, D, 0>(p, e, st);
-    if (p.bias_dtype == EVO_F32) return dq_ntw<T, D, 1>(p, e, st);
-    return dq_ntw<T, D, 2>(p, e, st);
+    return p.bias_dtype == EVO_NONE ? dq_ntw<T, D, false>(p, e, st) : dq_ntw<T, D, true>(p, e, st);
 }
 
 template <typename T, int D>
 static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned grid = (unsigned)((p.N + 127) / 128) * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, 0><<<grid, 256, 0, st>>>(p, e);
-    else if (p.bias_dtype == EVO_F32) mfma_dkdv<T, D, 1><<<grid, 256, 0, st>>>(p, e);
-    else mfma_dkdv<T, D, 2><<<grid, 256, 0, st>>>(p, e);
-    return hip_rc();
-}
-
-int EVO_CAT(launch_mfma_delta_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const int64_t rows = (int64_t)p.B * p.H * p.S * p.N;
-    const unsigned grid = (unsigned)((rows + 255) / 256);
-    if (p.dtype == EVO_BF16) mfma_delta<bf16_t, EVO_D><<<grid, 256, 0, st>>>(p, e.delta);
-    else mfma_delta<f16_t, EVO_D><<<grid, 256, 0, st>>>(p, e.delta);
+    if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false><<<grid, 256, 0, st>>>(p, e);
+    else mfma_dkdv<T, D, true><<<grid, 256, 0, st>>>(p, e);
     return hip_rc();
 }
 

@@ -6,12 +6,18 @@
 // input dtype before P.V (:84), LSE = m + log(l) and O = acc / l in the epilogue (:285-297).
 //
 // Tiling.  One workgroup = 4 waves = 128 query rows of one problem (b,h,s); each wave owns
-// 32 query rows for the whole key loop.  Keys are staged 64 at a time through LDS: K
+// 32 query rows for the whole key loop.  Keys are staged up to 256 at a time through LDS: K
 // row-major, V transposed.  The score tile is computed transposed, S^T = K Q^T, so that a
 // lane owns ONE query (column) and 16 keys (registers): the row max and row sum are
 // in-lane reductions plus a single exchange between the two lane groups, the rescale of
 // O^T is a per-lane scalar, and the probability tile in accumulator layout is already the
 // B operand of O^T = V^T P^T.
+//
+// The vector ALU, not the matrix core, bounds this kernel (one exp per score), so every
+// addition that can be moved into the matmul is: Q is pre-multiplied by scale*log2(e), the
+// bias tile (already in log2 units and accumulator order, see prep.hip) is the C operand of
+// the score MFMA, and the mask rides along as three extra columns of K against ones in Q.
+// What is left per score is max, subtract, exp2, add, convert.
 #include "common.h"
 #include "kernels.h"
 
@@ -21,25 +27,29 @@
 
 namespace evo {
 
-template <typename T, int D, int BIASK>
+template <typename T, int D, bool HAS_BIAS>
 __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
-    constexpr int BQ = 128, BKV = 64;
-    constexpr int DK = D < 16 ? 16 : D;  // contraction width of K Q^T, zero padded
-    constexpr int KS = DK / 16;
-    constexpr int DT = (D + 31) / 32;    // 32-row tiles of O^T
+    constexpr int BQ = 128;
+    constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round
+    constexpr int SPS = BKV / 64;                 // 64-key steps per stage
+    constexpr bool AUG_IN_PAD = D == 8;           // mask columns fit the zero padding of k-step 0
+    constexpr int KW = AUG_IN_PAD ? 16 : D + 16;  // K row: data, 3 mask columns, zeros
+    constexpr int KS = KW / 16;
+    constexpr int AUGC = AUG_IN_PAD ? 8 : D;
+    constexpr int DT = (D + 31) / 32;             // 32-row tiles of O^T
     constexpr int DP = DT * 32;
-    constexpr int KP = DK + 8;           // LDS pitches, padded against bank conflicts
+    constexpr int KP = KW + 8;                    // LDS pitches: conflict-free 16-byte reads
     constexpr int VP = BKV + 8;
+    constexpr float TAU = 8.0f;                   // rescale only when the max grows by > 2^TAU
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v2 v2;
 
     __shared__ __attribute__((aligned(16))) T Ks[BKV * KP];
     __shared__ __attribute__((aligned(16))) T Vt[DP * VP];
-    __shared__ __attribute__((aligned(16))) float Ms[BKV];
-    __shared__ float red[4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
+    const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nqb = (p.N + BQ - 1) / BQ;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nqb;
@@ -48,32 +58,43 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
     const int64_t sn = p.stride_n;
     const bool active = q0 < p.N;  // wave-uniform
+    const uint2 *m2row = e.m2 + ((int64_t)pr.b * p.S + pr.s) * npad;
+    const bool dead = e.dead[pr.b * p.S + pr.s] != 0;
 
-    // zero the LDS padding that is read but never staged (d >= D)
-    for (int i = tid; i < BKV * KP; i += 256) Ks[i] = (T)0.0f;
-    for (int i = tid; i < DP * VP; i += 256) Vt[i] = (T)0.0f;
+    // LDS that is read but never staged: the upper half of the mask k-step of K, rows d >= D
+    // of V^T
+    if (!AUG_IN_PAD)
+        for (int key = tid; key < BKV; key += 256)
+            *reinterpret_cast<v8 *>(&Ks[key * KP + AUGC + 8]) = zero8<T>();
+    if (DP > D)
+        for (int i = tid; i < (DP - D) * VP / 8; i += 256)
+            *reinterpret_cast<v8 *>(&Vt[D * VP + i * 8]) = zero8<T>();
 
-    // per-problem mask shift
-    float shift = 0.0f;
-    if (p.mask_kind != EVO_MASK_NONE) {
-        float mx = -INFINITY;
-        for (int j = tid; j < p.N; j += 256) mx = fmaxf(mx, mask_add(p, pr.b, pr.s, j));
-        mx = wave_max(mx);
-        if (lane == 0) red[wave] = mx;
-        __syncthreads();
-        shift = shift_from_max(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])));
-    }
-
+    // Q operand: data pre-multiplied by scale*log2(e); ones against the mask columns
     const int qrow = min(q0 + li, p.N - 1);
+    const float c = p.scale * kLog2e;
     v8 qf[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 16 + g * 8;
-        qf[ks] = d0 < D ? ld8(Q + (int64_t)qrow * sn + d0) : zero8<T>();
+        qf[ks] = zero8<T>();
+        if (d0 < D) {
+            if (!dead) {
+                v8 raw = ld8(Q + (int64_t)qrow * sn + d0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qf[ks][i] = (T)((float)raw[i] * c);
+            }
+        } else if (d0 == AUGC) {
+            qf[ks][0] = qf[ks][1] = qf[ks][2] = (T)1.0f;
+        }
     }
-    const int64_t brow = (int64_t)pr.b * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h + (int64_t)qrow * p.bias_stride_row;
-    const bool vec = e.vec_ok != 0;
-    const float scale = p.scale;
+
+    // bias tiles of this wave's query rows; a dead problem reads the all-zero tile instead
+    const int bb = e.bias_batches > 1 ? pr.b : 0;
+    const int qt = min(q0 >> 5, NT - 1);
+    const float *btile = dead ? e.bq + e.zero_tile + lane * 16
+                              : e.bq + ((((int64_t)bb * p.H + pr.h) * NT + qt) * NT) * 1024 + lane * 16;
+    const int64_t bstep = dead ? 0 : 1024;
 
     float m = -INFINITY, l = 0.0f;
     f32x16 oacc[DT];
@@ -82,86 +103,124 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
 
-    for (int kv0 = 0; kv0 < p.N; kv0 += BKV) {
+    // Bias tile kt into 16 registers; past the last tile the previous one is read again
+    // (every key there carries the mask floor, so the values do not matter).
+    auto load_btile = [&](int kt, f32x16 &dst) {
+        if (HAS_BIAS) {
+            const float *src = btile + (int64_t)min(kt, NT - 1) * bstep;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
+                dst[4 * rr] = v[0]; dst[4 * rr + 1] = v[1]; dst[4 * rr + 2] = v[2]; dst[4 * rr + 3] = v[3];
+            }
+        }
+    };
+
+    auto stage = [&](int kv0) {
         __syncthreads();  // readers of the previous stage are done
         for (int it = tid; it < BKV * (D / 8); it += 256) {
-            const int key = it / (D / 8), c = it % (D / 8), kk = kv0 + key;
-            v8 val = kk < p.N ? ld8(K + (int64_t)kk * sn + c * 8) : zero8<T>();
-            *reinterpret_cast<v8 *>(&Ks[key * KP + c * 8]) = val;
+            const int key = it / (D / 8), ch = it % (D / 8), kk = kv0 + key;
+            v8 val = kk < p.N ? ld8(K + (int64_t)kk * sn + ch * 8) : zero8<T>();
+            *reinterpret_cast<v8 *>(&Ks[key * KP + ch * 8]) = val;
         }
-        for (int it = tid; it < (BKV / 2) * (D / 8); it += 256) {
-            const int jp = it / (D / 8), c = it % (D / 8), k0 = kv0 + 2 * jp;
-            v8 a = k0 < p.N ? ld8(V + (int64_t)k0 * sn + c * 8) : zero8<T>();
-            v8 b = k0 + 1 < p.N ? ld8(V + (int64_t)(k0 + 1) * sn + c * 8) : zero8<T>();
+        for (int key = tid; key < BKV; key += 256) {
+            const int kk = kv0 + key;
+            const uint2 mv = kk < npad ? m2row[kk] : pack_split3<T>(kMaskFloor);
+            uint4 aug = {mv.x, mv.y, 0u, 0u};
+            *reinterpret_cast<uint4 *>(&Ks[key * KP + AUGC]) = aug;
+        }
+        constexpr int NPAIR = BKV / 2;
+        for (int it = tid; it < NPAIR * (D / 8); it += 256) {
+            const int ch = it / NPAIR, jp = it % NPAIR, k0 = kv0 + 2 * jp;
+            v8 a = k0 < p.N ? ld8(V + (int64_t)k0 * sn + ch * 8) : zero8<T>();
+            v8 b = k0 + 1 < p.N ? ld8(V + (int64_t)(k0 + 1) * sn + ch * 8) : zero8<T>();
             const int pos = perm_pos(2 * jp);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 v2 w;
                 w[0] = a[i];
                 w[1] = b[i];
-                *reinterpret_cast<v2 *>(&Vt[(c * 8 + i) * VP + pos]) = w;
+                *reinterpret_cast<v2 *>(&Vt[(ch * 8 + i) * VP + pos]) = w;
             }
         }
-        if (tid < BKV) Ms[tid] = mask_add(p, pr.b, pr.s, kv0 + tid);
         __syncthreads();
+    };
 
-        if (active) {
+    // One 64-key step: two score tiles, online softmax, four P.V k-steps.
+    auto compute = [&](int step, const f32x16 &c0, const f32x16 &c1) {
+        const int kb = (step % SPS) * 64;
+        f32x16 a0, a1;
 #pragma unroll
-            for (int kt = 0; kt < BKV / 32; ++kt) {
-                const int kb = kt * 32;
-                if (kv0 + kb >= p.N) break;
-                f32x16 acc;
+        for (int ks = 0; ks < KS; ++ks) {
+            v8 k0 = *reinterpret_cast<const v8 *>(&Ks[(kb + li) * KP + ks * 16 + g * 8]);
+            v8 k1 = *reinterpret_cast<const v8 *>(&Ks[(kb + 32 + li) * KP + ks * 16 + g * 8]);
+            if (ks == 0) {
+                if (HAS_BIAS) {
+                    a0 = Mfma<T>::mma(k0, qf[0], c0);
+                    a1 = Mfma<T>::mma(k1, qf[0], c1);
+                } else {
+                    f32x16 z;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    v8 a = *reinterpret_cast<const v8 *>(&Ks[(kb + li) * KP + ks * 16 + g * 8]);
-                    acc = Mfma<T>::mma(a, qf[ks], acc);
+                    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                    a0 = Mfma<T>::mma(k0, qf[0], z);
+                    a1 = Mfma<T>::mma(k1, qf[0], z);
                 }
-                float t[16];
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int kl = kb + 8 * rr + 4 * g, kg = kv0 + kl;
-                    float bv[4];
-                    load_bias4<BIASK, T>(p.bias, brow + kg, p.N - kg, vec, bv);
-                    const f32x4 mk = *reinterpret_cast<const f32x4 *>(&Ms[kl]);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) t[4 * rr + i] = fmaf(acc[4 * rr + i], scale, bv[i]) + mk[i];
-                }
-                if (shift != 0.0f) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) t[r] -= shift;
-                }
-                float mloc = t[0];
-#pragma unroll
-                for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, t[r]);
-                mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-                const float mn = fmaxf(fmaxf(m, mloc), -FLT_MAX);
-                const float alpha = fast_exp2((m - mn) * kLog2e);
-                float pv[16], psum = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    pv[r] = fast_exp2((t[r] - mn) * kLog2e);
-                    psum += pv[r];
-                }
-                l = l * alpha + psum;
-                m = mn;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-#pragma unroll
-                for (int ts = 0; ts < 2; ++ts) {
-                    v8 pf;
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) pf[i] = (T)pv[8 * ts + i];
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        v8 a = *reinterpret_cast<const v8 *>(&Vt[(dt * 32 + li) * VP + kb + ts * 16 + g * 8]);
-                        oacc[dt] = Mfma<T>::mma(a, pf, oacc[dt]);
-                    }
-                }
+            } else {
+                a0 = Mfma<T>::mma(k0, qf[ks], a0);
+                a1 = Mfma<T>::mma(k1, qf[ks], a1);
             }
+        }
+        float mloc = fmaxf(a0[0], a1[0]);
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+        const bool grow = mloc > m + TAU;
+        if (__any(grow)) {
+            const float mn = grow ? mloc : m;
+            const float alpha = fast_exp2(m - mn);
+            l *= alpha;
+            m = mn;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        }
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            a0[r] = fast_exp2(a0[r] - m);
+            a1[r] = fast_exp2(a1[r] - m);
+            psum += a0[r] + a1[r];
+        }
+        l += psum;
+#pragma unroll
+        for (int ts = 0; ts < 4; ++ts) {
+            v8 pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                v8 va = *reinterpret_cast<const v8 *>(&Vt[(dt * 32 + li) * VP + kb + ts * 16 + g * 8]);
+                oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
+            }
+        }
+    };
+
+    // Steps run in pairs on two register sets so that the bias tiles of the next step
+    // travel while the current one is computed, without register copies.
+    const int nsteps = (p.N + 63) / 64;
+    f32x16 tA0, tA1, tB0, tB1;
+    load_btile(0, tA0);
+    load_btile(1, tA1);
+    for (int step = 0; step < nsteps; step += 2) {
+        if (step % SPS == 0) stage(step * 64);
+        load_btile(2 * step + 2, tB0);
+        load_btile(2 * step + 3, tB1);
+        if (active) compute(step, tA0, tA1);
+        if (step + 1 < nsteps) {
+            load_btile(2 * step + 4, tA0);
+            load_btile(2 * step + 5, tA1);
+            if (active) compute(step + 1, tB0, tB1);
         }
     }
 
@@ -171,7 +230,8 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
         const int q = q0 + li;
         if (q < p.N) {
             T *O = (T *)p.o + pr.base + (int64_t)q * sn;
-            if (g == 0) p.lse[pr.row0 + q] = m + __logf(l);
+            // natural-log LSE of the (shifted) scores, as the reference stores it (:285-288)
+            if (g == 0) p.lse[pr.row0 + q] = (m + __log2f(l)) * kLn2;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -188,9 +248,8 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
 template <typename T, int D>
 static int fwd_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned nqb = (p.N + 127) / 128, grid = nqb * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, 0><<<grid, 256, 0, st>>>(p, e);
-    else if (p.bias_dtype == EVO_F32) mfma_fwd<T, D, 1><<<grid, 256, 0, st>>>(p, e);
-    else mfma_fwd<T, D, 2><<<grid, 256, 0, st>>>(p, e);
+    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, false><<<grid, 256, 0, st>>>(p, e);
+    else mfma_fwd<T, D, true><<<grid, 256, 0, st>>>(p, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }

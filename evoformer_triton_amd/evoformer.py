@@ -102,6 +102,10 @@ def _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
     return p
 
 
+def _alloc_bytes(nbytes, device):
+    return torch.empty((max(int(nbytes), 256),), device=device, dtype=torch.uint8)
+
+
 def _stream(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
@@ -130,8 +134,10 @@ def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
         O = torch.empty_like(Qc)                               # evoformer.py:654
         lse = torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32)   # :669-671
         p = _params(Qc, Kc, Vc, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
+        prep = _alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), Q.device)
+        p.prep, p.prep_bytes = _ptr(prep), prep.numel()
         _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(Q.device)), "evoattn_fwd")
-    ctx.save_for_backward(Qc, Kc, Vc, mask, bias, O, lse)       # :729
+    ctx.save_for_backward(Qc, Kc, Vc, mask, bias, O, lse, prep)  # :729
     ctx.layout = layout
     ctx.mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     ctx.bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
@@ -140,7 +146,7 @@ def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
 
 def _backward(ctx, dO, need_dmask, need_dbias):
     lib = _lib.load()
-    Q, K, V, mask, bias, O, lse = ctx.saved_tensors
+    Q, K, V, mask, bias, O, lse, prep = ctx.saved_tensors
     B, S, N, H, D = Q.shape
     mask_kind, mstr, mask_orig = ctx.mask_meta
     bias_dt, bstr, bias_orig = ctx.bias_meta
@@ -161,9 +167,10 @@ def _backward(ctx, dO, need_dmask, need_dbias):
         if want_dmask:
             dmask = torch.empty((B, S, N), device=Q.device, dtype=torch.float32)
             p.dmask = _ptr(dmask)
-        nbytes = lib.evoattn_bwd_workspace_bytes(ctypes.byref(p))
-        ws = torch.empty((max(int(nbytes), 1),), device=Q.device, dtype=torch.uint8)
-        p.workspace, p.workspace_bytes = _ptr(ws), int(nbytes)
+        ws = _alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), Q.device)
+        p.workspace, p.workspace_bytes = _ptr(ws), ws.numel()
+        p.prep, p.prep_bytes = _ptr(prep), prep.numel()
+        p.flags |= _lib.EVO_FLAG_PREP_VALID                      # same bias and mask as the forward
         _lib.check(lib.evoattn_bwd(ctypes.byref(p), _stream(Q.device)), "evoattn_bwd")
     if dbias is not None:
         shape, dtype = bias_orig

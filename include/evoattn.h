@@ -17,7 +17,7 @@
  *                   `_attn_bwd_preprocess` (:761-768), `_attn_bwd_dk_dv` (:776-812),
  *                   `_attn_bwd_dq` (:815-854), plus the zero-fill and the cast of
  *                   d_pair_bias (:752, :860)
- *   evoattn_bwd_workspace_bytes <- the `D = torch.empty_like(M)` and fp32 `d_pair_bias`
+ *   evoattn_prep_bytes, evoattn_bwd_workspace_bytes <- the `D = torch.empty_like(M)` and fp32 `d_pair_bias`
  *                   staging allocations (:752, :758), sized for the caller to make
  *   evoattn_check <- the asserts at :642-643 and :747-748
  */
@@ -52,7 +52,9 @@ enum {
 
 /* flags */
 enum {
-    EVO_FLAG_FORCE_GENERIC = 1  /* run the plain fp32-arithmetic kernels whatever the dtype */
+    EVO_FLAG_FORCE_GENERIC = 1, /* run the plain fp32-arithmetic kernels whatever the dtype */
+    EVO_FLAG_PREP_VALID    = 2  /* evoattn_bwd: `prep` still holds what evoattn_fwd wrote for the
+                                   same bias and mask; skip re-deriving it */
 };
 
 /* error codes */
@@ -105,6 +107,13 @@ typedef struct EvoAttnParams {
     float      *dmask;    /* dense [B][S][N] fp32 gradient of an additive mask, may be NULL */
     void       *workspace;
     size_t      workspace_bytes;
+
+    /* Prepared operands (bias in accumulator-tile order, mask rows in log2 units): scratch
+     * the matrix-core kernels derive from bias and mask at the start of evoattn_fwd.  The
+     * caller provides evoattn_prep_bytes() bytes, 256-byte aligned; it may hand the same
+     * buffer to evoattn_bwd with EVO_FLAG_PREP_VALID to skip the second derivation. */
+    void       *prep;
+    size_t      prep_bytes;
 } EvoAttnParams;
 
 int         evoattn_version(void);
@@ -112,6 +121,9 @@ const char *evoattn_strerror(int code);
 
 /* Host-only validation of a parameter block for one pass; launches nothing. */
 int evoattn_check(const EvoAttnParams *p, int pass);
+
+/* Bytes of the `prep` buffer evoattn_fwd and evoattn_bwd need (0 on invalid input). */
+size_t evoattn_prep_bytes(const EvoAttnParams *p);
 
 /* Bytes of device workspace evoattn_bwd needs for this problem (0 on invalid input). */
 size_t evoattn_bwd_workspace_bytes(const EvoAttnParams *p);

@@ -145,7 +145,8 @@ def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
 
     Oh = torch.empty_like(Qh)
     dQh, dKh, dVh = torch.empty_like(Qh), torch.empty_like(Qh), torch.empty_like(Qh)
-    lse = torch.empty((B, H, S, N), dtype=torch.float64 if Qh.dtype == torch.float64 else torch.float32)
+    lse = torch.empty((B, H, S, N), device=Qh.device,
+                      dtype=torch.float64 if Qh.dtype == torch.float64 else torch.float32)
     dbias = None if bias_h is None else torch.zeros_like(bias_h)
     dmask = torch.zeros_like(mask_h) if want_dmask else None
     for s0 in range(0, S, step):

@@ -1,0 +1,132 @@
+"""The C-ABI library loads on a GPU-less host, exports every symbol include/evoattn.h
+declares, and its host-side validation returns the documented codes.  No kernel runs."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from evoformer_triton_amd import _lib
+from evoformer_triton_amd._lib import EvoAttnParams
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(evoattn_\w+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = declared_functions()
+    assert set(names) == set(_lib.EXPORTS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.evoattn_version() == 1
+
+
+def test_struct_layout_matches_header():
+    # 12 x 4-byte fields, 9 x int64, 14 pointers, one size_t, then prep pointer + size; no padding
+    assert ctypes.sizeof(EvoAttnParams) == 12 * 4 + 9 * 8 + 14 * 8 + 8 + 16
+    assert EvoAttnParams.stride_b.offset == 48 and EvoAttnParams.q.offset == 120
+
+
+def good(B=1, S=4, N=64, H=2, D=32, dtype=_lib.EVO_BF16):
+    p = EvoAttnParams()
+    p.B, p.S, p.N, p.H, p.D = B, S, N, H, D
+    p.dtype, p.bias_dtype, p.mask_kind, p.dbias_dtype = dtype, _lib.EVO_F32, _lib.EVO_MASK_F32, _lib.EVO_F32
+    p.scale = D ** -0.5
+    p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * H * D, S * N * D, N * D, D
+    p.bias_stride_b, p.bias_stride_h, p.bias_stride_row = H * N * N, N * N, N
+    p.mask_stride_b, p.mask_stride_s = S * N, N
+    fake = 0x10000  # never dereferenced by the host-side checks
+    for f in ("q", "k", "v", "o", "lse", "bias", "mask", "dout", "dq", "dk", "dv", "dbias"):
+        setattr(p, f, fake)
+    p.workspace, p.workspace_bytes = fake, 1 << 30
+    p.prep, p.prep_bytes = fake, 1 << 30
+    return p
+
+
+def test_check_accepts_a_valid_block(lib):
+    p = good()
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == 0
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_FWD) == b"mfma"
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda p: setattr(p, "N", 0), _lib.EVO_EINVAL),
+    (lambda p: setattr(p, "q", None), _lib.EVO_EINVAL),
+    (lambda p: setattr(p, "dtype", 7), _lib.EVO_EINVAL),
+    (lambda p: setattr(p, "bias_dtype", _lib.EVO_F16), _lib.EVO_EINVAL),      # neither fp32 nor q's dtype
+    (lambda p: setattr(p, "bias", None), _lib.EVO_EINVAL),                    # dtype says there is one
+    (lambda p: setattr(p, "mask_kind", 9), _lib.EVO_EINVAL),
+    (lambda p: setattr(p, "scale", float("nan")), _lib.EVO_EINVAL),
+    (lambda p: setattr(p, "D", 24), _lib.EVO_EUNSUPPORTED),
+    (lambda p: setattr(p, "stride_n", 16), _lib.EVO_EINVAL),                  # rows would overlap
+    (lambda p: setattr(p, "q", 0x10001), _lib.EVO_EALIGN),
+    (lambda p: setattr(p, "lse", 0x10002), _lib.EVO_EALIGN),
+    (lambda p: setattr(p, "B", 1 << 30), _lib.EVO_EOVERFLOW),
+])
+def test_check_rejects(lib, mutate, code):
+    p = good()
+    mutate(p)
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == code
+    assert lib.evoattn_fwd(ctypes.byref(p), None) == code      # rejected before any launch
+    assert lib.evoattn_strerror(code)
+
+
+def test_bwd_checks_workspace_and_outputs(lib):
+    p = good()
+    need = lib.evoattn_bwd_workspace_bytes(ctypes.byref(p))
+    rows = 1 * 2 * 4 * 64
+    assert need >= rows * 4 + 4 * 4 + 2 * 64 * 64 * 4          # delta + shift + >= one dBias partial
+    p.workspace_bytes = need - 1
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EWORKSPACE
+    p.workspace_bytes = need
+    p.workspace = 0x10010
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EALIGN
+    p = good()
+    p.dq = None
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL
+    assert lib.evoattn_bwd(ctypes.byref(p), None) == _lib.EVO_EINVAL
+    p = good()
+    p.dbias_dtype = _lib.EVO_F16
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL
+    # without dbias / dmask the workspace shrinks
+    p = good()
+    p.dbias = None
+    assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) < need
+    assert lib.evoattn_bwd_workspace_bytes(None) == 0
+
+
+def test_path_selection(lib):
+    p = good(dtype=_lib.EVO_F32)
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"            # check mode
+    p = good(D=128)
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"
+    p = good()
+    p.flags = _lib.EVO_FLAG_FORCE_GENERIC
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"
+    p = good()
+    p.q = 0x10008                                                          # 8-byte aligned only
+    assert lib.evoattn_check(ctypes.byref(p), 0) == 0
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"
+    p = good(N=4096)
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"mfma"
+    assert lib.evoattn_path(ctypes.byref(p), 1) == b"generic"            # dBias tiles exceed the register file
+
+
+def test_error_strings(lib):
+    assert _lib.strerror(0) == "ok"
+    assert "workspace" in _lib.strerror(_lib.EVO_EWORKSPACE)
+    assert _lib.strerror(_lib.EVO_EHIP - 1)                                # a hipError_t string
+    with pytest.raises(_lib.EvoAttnError) as ei:
+        _lib.check(_lib.EVO_EALIGN, "evoattn_fwd")
+    assert ei.value.code == _lib.EVO_EALIGN and "evoattn_fwd" in str(ei.value)

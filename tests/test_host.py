@@ -1,0 +1,90 @@
+"""Host-side logic of the autograd boundary that needs no GPU: stride maps of the two head
+layouts, mask / bias canonicalisation, argument errors, and the loud failure on CPU tensors
+(there is no CPU implementation behind the operator)."""
+import pytest
+import torch
+
+import evoformer_triton_amd.evoformer as E
+from evoformer_triton_amd import _lib
+
+
+def test_reference_strides_are_the_flat_reshape():
+    B, S, N, H, D = 2, 3, 5, 4, 8
+    x = torch.arange(B * S * N * H * D).reshape(B, S, N, H, D)
+    sb, sh, ss, sn = E._q_strides(B, S, N, H, D, "reference")
+    view = x.reshape(B, H, S, N, D)            # evoformer.py:648-650
+    flat = x.reshape(-1)
+    for b, h, s, n in ((0, 0, 0, 0), (1, 3, 2, 4), (0, 2, 1, 3)):
+        assert torch.equal(flat[b * sb + h * sh + s * ss + n * sn: b * sb + h * sh + s * ss + n * sn + D], view[b, h, s, n])
+    sb, sh, ss, sn = E._q_strides(B, S, N, H, D, "ds4sci")
+    perm = x.permute(0, 3, 1, 2, 4)
+    for b, h, s, n in ((0, 0, 0, 0), (1, 3, 2, 4), (0, 2, 1, 3)):
+        off = b * sb + h * sh + s * ss + n * sn
+        assert torch.equal(flat[off: off + D], perm[b, h, s, n])
+    with pytest.raises(ValueError):
+        E._q_strides(B, S, N, H, D, "nope")
+
+
+def test_mask_canonicalisation():
+    dev = torch.device("cpu")
+    m, kind, st = E._prep_mask(None, 2, 3, 5, dev)
+    assert m is None and kind == _lib.EVO_MASK_NONE
+    m, kind, st = E._prep_mask(torch.ones(2, 3, 1, 1, 5, dtype=torch.bool), 2, 3, 5, dev)
+    assert kind == _lib.EVO_MASK_BOOL and st == (15, 5)
+    m, kind, st = E._prep_mask(torch.zeros(1, 3, 1, 1, 5), 2, 3, 5, dev)
+    assert kind == _lib.EVO_MASK_F32 and st == (0, 5)                      # broadcast over B
+    m, kind, st = E._prep_mask(torch.zeros(2, 1, 1, 1, 5, dtype=torch.bfloat16), 2, 3, 5, dev)
+    assert kind == _lib.EVO_MASK_BF16 and st == (5, 0)                     # broadcast over S
+    m, kind, st = E._prep_mask(torch.zeros(2, 3, 1, 1, 5, dtype=torch.float64), 2, 3, 5, dev)
+    assert kind == _lib.EVO_MASK_F32 and m.dtype == torch.float32
+    m, kind, st = E._prep_mask(torch.ones(2, 3, 1, 1, 5, dtype=torch.int64), 2, 3, 5, dev)
+    assert kind == _lib.EVO_MASK_BOOL and m.dtype == torch.bool
+    with pytest.raises(ValueError):
+        E._prep_mask(torch.zeros(2, 3, 1, 5), 2, 3, 5, dev)
+    with pytest.raises(ValueError):
+        E._prep_mask(torch.zeros(2, 3, 1, 1, 6), 2, 3, 5, dev)
+
+
+def test_bias_canonicalisation():
+    dev = torch.device("cpu")
+    b, dt, st = E._prep_bias(None, 2, 4, 5, torch.bfloat16, dev)
+    assert b is None and dt == _lib.EVO_NONE
+    b, dt, st = E._prep_bias(torch.zeros(2, 1, 4, 5, 5), 2, 4, 5, torch.bfloat16, dev)
+    assert dt == _lib.EVO_F32 and st == (100, 25, 5)
+    b, dt, st = E._prep_bias(torch.zeros(1, 1, 4, 5, 5, dtype=torch.bfloat16), 2, 4, 5, torch.bfloat16, dev)
+    assert dt == _lib.EVO_BF16 and st == (0, 25, 5)
+    b, dt, st = E._prep_bias(torch.zeros(2, 1, 4, 5, 5, dtype=torch.float16), 2, 4, 5, torch.bfloat16, dev)
+    assert dt == _lib.EVO_F32 and b.dtype == torch.float32                  # foreign 16-bit type is widened
+    nc = torch.zeros(2, 1, 4, 5, 10)[..., ::2]
+    b, dt, st = E._prep_bias(nc, 2, 4, 5, torch.float32, dev)
+    assert b.is_contiguous()
+    with pytest.raises(ValueError):
+        E._prep_bias(torch.zeros(2, 4, 5, 5), 2, 4, 5, torch.float32, dev)
+
+
+def test_argument_errors_and_no_cpu_fallback():
+    q = torch.zeros(1, 2, 8, 2, 8, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        E.EvoformerAttention.apply(q, q, q, None, None)
+    with pytest.raises(AssertionError):
+        E.EvoformerAttention.apply(q, q, torch.zeros(1, 2, 8, 2, 16, dtype=torch.bfloat16), None, None)
+    with pytest.raises(TypeError):
+        E.EvoformerAttention.apply(q.double(), q.double(), q.double(), None, None)
+    with pytest.raises(ValueError):
+        E.EvoformerAttention.apply(q[0], q[0], q[0], None, None)
+    with pytest.raises(ValueError):
+        E.DS4Sci_EvoformerAttention(q, q, q, [None, None, None])
+    with pytest.raises(TypeError):
+        E.DS4Sci_EvoformerAttention(q, q, q, [torch.ones(1, 2, 1, 1, 8, dtype=torch.bool)])
+    with pytest.raises(ValueError):
+        E.evoformer_attention(q, q, q, None, None, layout="x")
+
+
+def test_drop_in_module_name():
+    import evoformer
+    assert evoformer.EvoformerAttention is E.EvoformerAttention
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load(str(tmp_path / "libevoattn.so"))
