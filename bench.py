@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Benchmark of the Evoformer attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2]
+
+One "step" is one forward + backward of the attention over one batch of synthetic input
+(BASELINE configuration C2 by default: MSA row attention, Q,K,V [1,512,256,8,32] bf16,
+additive row mask, bf16 pair bias), called through the public operator
+`EvoformerAttention.apply` + autograd, inputs resident in HBM.  Prints ONE JSON line.
+
+`value` is algorithmic TFLOP/s: 14*B*S*H*N^2*D per step (the reference's convention,
+speed_benchmark.py:109-115, with the S factor its S=1 benchmark omits) over the measured
+time per step.  `roofline` prices the slowest kernel of the step against the MI355X dense
+bf16 MFMA peak; its duration is measured here with HIP events around back-to-back launches
+of that kernel alone on the launch stream.  `cpu_baseline` is the eager oracle timed on the
+host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="C2", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, shape, budget_s=15.0):
+    """The eager oracle (fp32, chunked over S) on the host cores, on a slice of S rows."""
+    import torch
+    from oracle import eager
+    B, S, N, H, D = shape
+    threads = torch.get_num_threads()
+    s_sample = S if cfg in ("C2", "C3") else max(1, S // 8)   # whole workload where it takes well under a second
+    x = eager.make_inputs(cfg, shape=(B, s_sample, N, H, D))
+
+    def once():
+        t0 = time.perf_counter()
+        eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"],
+                                compute_dtype=torch.float32, s_chunk=8)
+        return time.perf_counter() - t0
+
+    warm = once()
+    reps = int(max(1, min(20, budget_s / max(warm, 1e-3))))
+    t = statistics.median(once() for _ in range(reps))
+    flops = eager.flops_fwd_bwd(B, s_sample, N, H, D)[2]
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{s_sample} of {S} S-rows of {cfg} ({s_sample / S:.4f} of the workload), eager fp32 oracle "
+                      f"chunked 8 rows at a time, 1 warm-up + median of {reps} runs, {t:.3f} s per run"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
+              "(the path shards over S with one dBias all-reduce, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from oracle import eager
+    import evoformer_triton_amd.evoformer as E
+    from evoformer_triton_amd import EvoformerAttention, _lib
+
+    lib = _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    x = eager.make_inputs(args.config)
+    B, S, N, H, D = x["shape"]
+    q, k, v = (x[n].to(dev).requires_grad_() for n in "QKV")
+    bias = x["bias"].to(dev).requires_grad_()
+    mask, dO = x["mask"].to(dev), x["dO"].to(dev)
+    f_fwd, f_bwd, f_full = eager.flops_fwd_bwd(B, S, N, H, D)
+
+    def step():
+        o = EvoformerAttention.apply(q, k, v, mask, bias)
+        return torch.autograd.grad(o, (q, k, v, bias), dO)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base_mem = torch.cuda.memory_allocated()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    peak_extra = torch.cuda.max_memory_allocated() - base_mem
+
+    # ---- kernel-level timing through the C ABI, buffers preallocated
+    qc, kc, vc = q.detach(), k.detach(), v.detach()
+    m, mk, mstr = E._prep_mask(mask, B, S, N, dev)
+    bz, bdt, bstr = E._prep_bias(bias.detach(), B, H, N, qc.dtype, dev)
+    o = torch.empty_like(qc)
+    lse = torch.empty((B, H, S, N), device=dev)
+    p = E._params(qc, kc, vc, m, mk, mstr, bz, bdt, bstr, o, lse, "reference")
+    prep = E._alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), dev)
+    p.prep, p.prep_bytes = prep.data_ptr(), prep.numel()
+    dq, dk, dv = (torch.empty_like(qc) for _ in range(3))
+    dbias = torch.empty((B, H, N, N), device=dev, dtype=bz.dtype)
+    p.dout, p.dq, p.dk, p.dv, p.dbias = dO.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dbias.data_ptr()
+    p.dbias_dtype = E._DTYPES[bz.dtype]
+    ws = E._alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), dev)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, n):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e-3
+
+    def call(fn, flags):
+        p.flags = flags
+        rc = fn(ctypes.byref(p), st)
+        assert rc == 0, _lib.strerror(rc)
+
+    V = _lib.EVO_FLAG_PREP_VALID
+    phases = {
+        "fwd": (lambda: call(lib.evoattn_fwd, 0), f_fwd),
+        "bwd_dq": (lambda: call(lib.evoattn_bwd, V | _lib.EVO_FLAG_ONLY_DQ), f_bwd / 2),
+        "bwd_dkdv": (lambda: call(lib.evoattn_bwd, V | _lib.EVO_FLAG_ONLY_DKDV), f_bwd / 2),
+    }
+    call(lib.evoattn_fwd, 0)
+    call(lib.evoattn_bwd, V)
+    n_k = max(10, args.steps)
+    t_phase = {name: timed(fn, n_k) for name, (fn, _) in phases.items()}
+    t_abi = timed(lambda: (call(lib.evoattn_fwd, 0), call(lib.evoattn_bwd, V)), n_k)
+    dom = max(t_phase, key=t_phase.get)
+    achieved = phases[dom][1] / t_phase[dom] / 1e12
+    kernel_names = {"fwd": "mfma_fwd", "bwd_dq": "mfma_dq", "bwd_dkdv": "mfma_dkdv"}
+
+    esz = qc.element_size()
+    io_bytes = 12 * qc.numel() * esz + 2 * bias.numel() * bias.element_size()   # algorithmic HBM bytes per step
+    out = {
+        "metric": "fwd+bwd TFLOP/s (S=%d N=%d H=%d D=%d)" % (S, N, H, D),
+        "value": f_full / dt / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.config}: Evoformer attention fwd+bwd through EvoformerAttention.apply + autograd, "
+                               f"Q,K,V [B={B},S={S},N={N},H={H},D={D}] bf16, additive row mask [{B},{S},1,1,{N}], "
+                               f"pair bias [{B},1,{H},{N},{N}] bf16, seeded N(0,1) inputs",
+                   "flops_per_step": f_full, "algorithmic_hbm_bytes_per_step": io_bytes},
+        "pct_mfma_peak": 100.0 * f_full / dt / 1e12 / MFMA_PEAK_TFLOPS,
+        "pct_hbm_peak": 100.0 * io_bytes / dt / 1e9 / HBM_PEAK_GBS,
+        "fwd_tflops": f_fwd / t_phase["fwd"] / 1e12,
+        "c_abi_ms_per_step": t_abi * 1e3,
+        "c_abi_tflops": f_full / t_abi / 1e12,
+        "kernel_ms": {kernel_names[n]: t * 1e3 for n, t in t_phase.items()},
+        "peak_mem_bytes_beyond_inputs": int(peak_extra),
+        "roofline": {"bound": "mfma", "kernel": kernel_names[dom], "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+                     "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.config, (B, S, N, H, D))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

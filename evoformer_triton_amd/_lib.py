@@ -16,6 +16,8 @@ EVO_NONE, EVO_BF16, EVO_F16, EVO_F32 = -1, 0, 1, 2
 EVO_MASK_NONE, EVO_MASK_BOOL, EVO_MASK_F32, EVO_MASK_BF16, EVO_MASK_F16 = 0, 1, 2, 3, 4
 EVO_FLAG_FORCE_GENERIC = 1
 EVO_FLAG_PREP_VALID = 2
+EVO_FLAG_ONLY_DQ = 4
+EVO_FLAG_ONLY_DKDV = 8
 EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 

@@ -216,6 +216,8 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     if ((rc = check_prep(*p))) return rc;
     fill_prep(*p, e);
     if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
+    if (p->flags & EVO_FLAG_ONLY_DQ) return launch_mfma_dq(*p, e, st);
+    if (p->flags & EVO_FLAG_ONLY_DKDV) return launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads
     if ((rc = launch_mfma_dq(*p, e, st))) return rc;
     if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;

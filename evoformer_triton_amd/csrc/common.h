@@ -173,6 +173,18 @@ __device__ __forceinline__ void split3<f16_t>(float m, f16_t &hi, f16_t &mid, f1
     lo = (f16_t)(r1 - (float)mid);
 }
 
+// raw * c as hi + lo, both representable in T: the product to 16 significant bits.
+template <typename T>
+__device__ __forceinline__ void scaled_hilo8(typename Mfma<T>::v8 raw, float c, typename Mfma<T>::v8 &hi,
+                                             typename Mfma<T>::v8 &lo) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float f = (float)raw[i] * c;
+        hi[i] = (T)f;
+        lo[i] = (T)(f - (float)hi[i]);
+    }
+}
+
 // (hi, mid, lo, 0) of split3 packed into 8 bytes.
 template <typename T>
 __device__ __forceinline__ uint2 pack_split3(float m) {

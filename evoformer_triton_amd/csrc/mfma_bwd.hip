@@ -41,6 +41,10 @@ struct Geo {
     static constexpr int AUGC = AUG_IN_PAD ? 8 : D;      // first extra column
     static constexpr int DT = (D + 31) / 32;
     static constexpr int DP = DT * 32;
+    // The operand scaled by scale*log2(e) is rounded to 16 bits; for small head dims, where
+    // the matrix core has k-steps to spare, its rounding residue is carried as well, which
+    // makes the scores exact to fp32 (and identical in the forward and both backward kernels).
+    static constexpr bool RESID = D <= 16;
 };
 
 template <typename T>
@@ -156,8 +160,10 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
         const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
 
         // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
-        v8 qf[KS], gf[KS];
+        v8 qf[KS], gf[KS], qlo[KSD];
         float dpart = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KSD; ++ks) qlo[ks] = zero8<T>();
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int d0 = ks * 16 + g * 8;
@@ -167,7 +173,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
                 v8 qraw = ld8(Q + (int64_t)qrow * sn + d0);
                 gf[ks] = ld8(Gd + (int64_t)qrow * sn + d0);
                 v8 oraw = ld8(O + (int64_t)qrow * sn + d0);
-                if (!dead) qf[ks] = scaled8<T>(qraw, cs);
+                if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) dpart = fmaf((float)gf[ks][i], (float)oraw[i], dpart);
             }
@@ -238,6 +244,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     acc = Mfma<T>::mma(ka[ks], qf[ks], acc);   // log2 P^T
+                    if (G::RESID && ks < KSD) acc = Mfma<T>::mma(ka[ks], qlo[ks], acc);
                     dp = Mfma<T>::mma(va[ks], gf[ks], dp);     // dP^T - delta
                 }
                 float ds[16];
@@ -336,11 +343,12 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 template <typename T, int D, bool HAS_BIAS>
 __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
-    constexpr int KW = G::KW, KS = G::KS, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
+    constexpr int KW = G::KW, KS = G::KS, KSD = G::KSD, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
     constexpr int BK = 128;
     constexpr int BQS = D <= 32 ? 128 : 64;  // query rows staged per round
     constexpr int TPS = BQS / 32;            // query tiles per stage
-    constexpr int QP = KW + 8;
+    constexpr int RW = G::RESID ? KSD * 16 : 0;  // residue columns of the scaled Q rows
+    constexpr int QP = KW + RW + 8;
     constexpr int TP = BQS + 8;
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v2 v2;
@@ -376,6 +384,8 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
             *reinterpret_cast<v8 *>(&Qs[r * QP + AUGC + 8]) = zero8<T>();
             *reinterpret_cast<v8 *>(&Gs[r * QP + AUGC + 8]) = zero8<T>();
         }
+    if (G::RESID && D < 16)
+        for (int r = tid; r < BQS; r += 256) *reinterpret_cast<v8 *>(&Qs[r * QP + KW + 8]) = zero8<T>();
     if (DP > D)
         for (int i = tid; i < (DP - D) * TP / 8; i += 256) {
             *reinterpret_cast<v8 *>(&Qt[D * TP + i * 8]) = zero8<T>();
@@ -383,7 +393,9 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
         }
 
     // this wave's keys: K with the mask columns, V with ones against -delta
-    v8 kf[KS], vf[KS];
+    v8 kf[KS], vf[KS], kres[KSD];
+#pragma unroll
+    for (int ks = 0; ks < KSD; ++ks) kres[ks] = zero8<T>();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 16 + g * 8;
@@ -391,6 +403,7 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
         vf[ks] = zero8<T>();
         if (d0 < D) {
             if (!dead) kf[ks] = ld8(K + (int64_t)keyc * sn + d0);
+            if (ks < KSD) kres[ks] = kf[ks];   // against the residue columns of Q: data only
             vf[ks] = ld8(V + (int64_t)keyc * sn + d0);
         } else if (d0 == AUGC) {
             const int kk = min(key, npad - 1);
@@ -429,7 +442,10 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
             v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + ch * 8) : zero8<T>();
             v8 bb2 = qq < p.N ? ld8(Gd + (int64_t)qq * sn + ch * 8) : zero8<T>();
             // the score operand carries scale*log2(e), rounded exactly as in the forward
-            *reinterpret_cast<v8 *>(&Qs[row * QP + ch * 8]) = scaled8<T>(a, cs);
+            v8 hi, lo;
+            scaled_hilo8<T>(a, cs, hi, lo);
+            *reinterpret_cast<v8 *>(&Qs[row * QP + ch * 8]) = hi;
+            if (G::RESID) *reinterpret_cast<v8 *>(&Qs[row * QP + KW + ch * 8]) = lo;
             *reinterpret_cast<v8 *>(&Gs[row * QP + ch * 8]) = bb2;
         }
         for (int row = tid; row < BQS; row += 256) {
@@ -483,6 +499,13 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
                 acc = Mfma<T>::mma(qa, kf[ks], acc);           // log2 P
             }
             dp = Mfma<T>::mma(ga, vf[ks], dp);                 // dP - delta
+        }
+        if (G::RESID) {
+#pragma unroll
+            for (int ks = 0; ks < KSD; ++ks) {
+                v8 ql = *reinterpret_cast<const v8 *>(&Qs[(qb + li) * QP + KW + ks * 16 + g * 8]);
+                acc = Mfma<T>::mma(ql, kres[ks], acc);
+            }
         }
         float ds[16];
 #pragma unroll

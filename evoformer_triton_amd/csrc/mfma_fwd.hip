@@ -41,6 +41,11 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
     constexpr int KP = KW + 8;                    // LDS pitches: conflict-free 16-byte reads
     constexpr int VP = BKV + 8;
     constexpr float TAU = 8.0f;                   // rescale only when the max grows by > 2^TAU
+    // Q * scale * log2(e) is rounded to 16 bits; where the matrix core has k-steps to spare
+    // (small head dims) the rounding residue rides along as a second operand, which makes
+    // the scores exact to fp32.
+    constexpr bool RESID = D <= 16;
+    constexpr int KSD = (D + 15) / 16;
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v2 v2;
 
@@ -73,17 +78,15 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
     // Q operand: data pre-multiplied by scale*log2(e); ones against the mask columns
     const int qrow = min(q0 + li, p.N - 1);
     const float c = p.scale * kLog2e;
-    v8 qf[KS];
+    v8 qf[KS], qlo[KSD];
+#pragma unroll
+    for (int ks = 0; ks < KSD; ++ks) qlo[ks] = zero8<T>();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         const int d0 = ks * 16 + g * 8;
         qf[ks] = zero8<T>();
         if (d0 < D) {
-            if (!dead) {
-                v8 raw = ld8(Q + (int64_t)qrow * sn + d0);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) qf[ks][i] = (T)((float)raw[i] * c);
-            }
+            if (!dead) scaled_hilo8<T>(ld8(Q + (int64_t)qrow * sn + d0), c, qf[ks], qlo[ks < KSD ? ks : 0]);
         } else if (d0 == AUGC) {
             qf[ks][0] = qf[ks][1] = qf[ks][2] = (T)1.0f;
         }
@@ -168,6 +171,10 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
             } else {
                 a0 = Mfma<T>::mma(k0, qf[ks], a0);
                 a1 = Mfma<T>::mma(k1, qf[ks], a1);
+            }
+            if (RESID && ks < KSD) {
+                a0 = Mfma<T>::mma(k0, qlo[ks], a0);
+                a1 = Mfma<T>::mma(k1, qlo[ks], a1);
             }
         }
         float mloc = fmaxf(a0[0], a1[0]);

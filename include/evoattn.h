@@ -53,8 +53,13 @@ enum {
 /* flags */
 enum {
     EVO_FLAG_FORCE_GENERIC = 1, /* run the plain fp32-arithmetic kernels whatever the dtype */
-    EVO_FLAG_PREP_VALID    = 2  /* evoattn_bwd: `prep` still holds what evoattn_fwd wrote for the
+    EVO_FLAG_PREP_VALID    = 2, /* evoattn_bwd: `prep` still holds what evoattn_fwd wrote for the
                                    same bias and mask; skip re-deriving it */
+    /* Measurement aids: enqueue a single phase of the matrix-core backward.  ONLY_DQ runs
+     * the dQ kernel (dq, delta and the dBias partials, no final dBias sum); ONLY_DKDV runs
+     * the dK/dV kernel and needs the delta a previous full call left in the same workspace. */
+    EVO_FLAG_ONLY_DQ       = 4,
+    EVO_FLAG_ONLY_DKDV     = 8
 };
 
 /* error codes */

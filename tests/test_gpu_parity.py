@@ -370,15 +370,21 @@ def test_benchmark_configs_full_size(E, cfg):
                                       compute_dtype=torch.float32)
     got = run_hip(E, x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], mask_grad=True)
     main = ("O", "dQ", "dK", "dV")
+    e_f32 = {n: max_err(got[n], ref_f32[n]) for n in main}
+    e_bf = {n: max_err(got[n], ref_bf16[n]) for n in main}
+    e_self = {n: max_err(ref_bf16[n], ref_f32[n]) for n in main}
+    mags = {n: ref_f32[n].abs().max().item() for n in main}
+    print(f"\n{cfg}: max-abs vs eager-fp32 {e_f32} | vs eager-bf16 {e_bf} | eager-bf16 vs eager-fp32 {e_self} | max|ref| {mags}")
     # (1) against the exact value of the eager formula on the same bf16 inputs (fp32 eager)
-    e_f32 = assert_close(got, ref_f32, FULL_TOL[cfg], main, what=f"{cfg} vs eager fp32")
+    # C5 (D=8, N=384) has |dK| up to 5.5 and |dQ| up to 3.3, where the rounding of the bf16
+    # result alone is 1.6e-2 / 0.8e-2: there the bound is the tolerance plus half a bf16
+    # ulp of the entry (the output rounding itself); eager in bf16 is 5.3e-2 away.
+    assert_close(got, ref_f32, FULL_TOL[cfg], main, what=f"{cfg} vs eager fp32",
+                 ulp_names=("dQ", "dK", "dV") if cfg == "C5" else (), ulps=0.5)
     # (2) against eager run as the reference writes it, all in bf16.  With a bf16 bias its
     # scores are themselves rounded to bf16 (test.py:53), so it sits up to e_self away from
     # the exact value; the HIP result must be within the tolerance of it once that is allowed.
-    e_bf, e_self = {}, {}
     for n in main:
-        e_bf[n] = max_err(got[n], ref_bf16[n])
-        e_self[n] = max_err(ref_bf16[n], ref_f32[n])
         assert e_bf[n] <= FULL_TOL[cfg] + e_self[n], f"{cfg} {n}: {e_bf[n]:.3e} vs eager bf16 (its own error {e_self[n]:.3e})"
     # dBias (a sum of dS over S rows) and dMask (over heads and queries) reach |x| ~ 15..25
     # here and come back in bf16, where one ulp is 6e-2..1.2e-1: an absolute 2e-2 cannot
@@ -391,7 +397,7 @@ def test_benchmark_configs_full_size(E, cfg):
         e_self[n] = max_err(ref_bf16[n], ref_f32[n])
         atol = FULL_REDUCED_ATOL if n == "dBias" else FULL_DMASK_ATOL
         assert torch.allclose(a, b, atol=atol, rtol=1e-2), f"{n} max-abs {e_f32[n]:.3e} (|ref| max {b.abs().max().item():.2f})"
-    print(f"\n{cfg}: max-abs vs eager-fp32 {e_f32} | vs eager-bf16 {e_bf} | eager-bf16 vs eager-fp32 {e_self}")
+    print(f"{cfg}: reduced gradients max-abs vs eager-fp32 { {n: e_f32[n] for n in ('dBias', 'dMask')} } | eager-bf16's own { {n: e_self[n] for n in ('dBias', 'dMask')} }")
 
 
 def test_full_size_properties_c2(E):
