@@ -5,8 +5,8 @@
 // and mask fused before the running max (:68-71), online softmax (:71-89), P cast to the
 // input dtype before P.V (:84), LSE = m + log(l) and O = acc / l in the epilogue (:285-297).
 //
-// Tiling.  One workgroup = 4 waves = 128 query rows of one problem (b,h,s); each wave owns
-// 32 query rows for the whole key loop.  Keys are staged up to 256 at a time through LDS: K
+// Tiling.  One workgroup = NW (4 or 8) waves = NW*32 query rows of one problem (b,h,s); each
+// wave owns 32 query rows for the whole key loop.  Keys are staged up to 256 at a time through LDS: K
 // row-major, V transposed.  The score tile is computed transposed, S^T = K Q^T, so that a
 // lane owns ONE query (column) and 16 keys (registers): the row max and row sum are
 // in-lane reductions plus a single exchange between the two lane groups, the rescale of
@@ -27,9 +27,10 @@
 
 namespace evo {
 
-template <typename T, int D, bool HAS_BIAS>
-__global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
-    constexpr int BQ = 128;
+template <typename T, int D, bool HAS_BIAS, int NW>
+__global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_fwd(EvoAttnParams p, Extra e) {
+    constexpr int NTH = NW * 64;                  // threads per workgroup
+    constexpr int BQ = NW * 32;                   // query rows per workgroup
     constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round
     constexpr int SPS = BKV / 64;                 // 64-key steps per stage
     constexpr bool AUG_IN_PAD = D == 8;           // mask columns fit the zero padding of k-step 0
@@ -69,10 +70,10 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
     // LDS that is read but never staged: the upper half of the mask k-step of K, rows d >= D
     // of V^T
     if (!AUG_IN_PAD)
-        for (int key = tid; key < BKV; key += 256)
+        for (int key = tid; key < BKV; key += NTH)
             *reinterpret_cast<v8 *>(&Ks[key * KP + AUGC + 8]) = zero8<T>();
     if (DP > D)
-        for (int i = tid; i < (DP - D) * VP / 8; i += 256)
+        for (int i = tid; i < (DP - D) * VP / 8; i += NTH)
             *reinterpret_cast<v8 *>(&Vt[D * VP + i * 8]) = zero8<T>();
 
     // Q operand: data pre-multiplied by scale*log2(e); ones against the mask columns
@@ -121,19 +122,19 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
 
     auto stage = [&](int kv0) {
         __syncthreads();  // readers of the previous stage are done
-        for (int it = tid; it < BKV * (D / 8); it += 256) {
+        for (int it = tid; it < BKV * (D / 8); it += NTH) {
             const int key = it / (D / 8), ch = it % (D / 8), kk = kv0 + key;
             v8 val = kk < p.N ? ld8(K + (int64_t)kk * sn + ch * 8) : zero8<T>();
             *reinterpret_cast<v8 *>(&Ks[key * KP + ch * 8]) = val;
         }
-        for (int key = tid; key < BKV; key += 256) {
+        for (int key = tid; key < BKV; key += NTH) {
             const int kk = kv0 + key;
             const uint2 mv = kk < npad ? m2row[kk] : pack_split3<T>(kMaskFloor);
             uint4 aug = {mv.x, mv.y, 0u, 0u};
             *reinterpret_cast<uint4 *>(&Ks[key * KP + AUGC]) = aug;
         }
         constexpr int NPAIR = BKV / 2;
-        for (int it = tid; it < NPAIR * (D / 8); it += 256) {
+        for (int it = tid; it < NPAIR * (D / 8); it += NTH) {
             const int ch = it / NPAIR, jp = it % NPAIR, k0 = kv0 + 2 * jp;
             v8 a = k0 < p.N ? ld8(V + (int64_t)k0 * sn + ch * 8) : zero8<T>();
             v8 b = k0 + 1 < p.N ? ld8(V + (int64_t)(k0 + 1) * sn + ch * 8) : zero8<T>();
@@ -149,8 +150,10 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
         __syncthreads();
     };
 
-    // One 64-key step: two score tiles, online softmax, four P.V k-steps.
-    auto compute = [&](int step, const f32x16 &c0, const f32x16 &c1) {
+    // One 64-key step: two score tiles, online softmax, four P.V k-steps.  The bias tiles
+    // c0, c1 are consumed by the first score MFMAs; the same registers then receive the
+    // tiles of the next step, which travel while the softmax and P.V run.
+    auto compute = [&](int step, f32x16 &c0, f32x16 &c1) {
         const int kb = (step % SPS) * 64;
         f32x16 a0, a1;
 #pragma unroll
@@ -177,6 +180,8 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
                 a1 = Mfma<T>::mma(k1, qlo[ks], a1);
             }
         }
+        load_btile(2 * step + 2, c0);
+        load_btile(2 * step + 3, c1);
         float mloc = fmaxf(a0[0], a1[0]);
 #pragma unroll
         for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
@@ -213,22 +218,13 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
         }
     };
 
-    // Steps run in pairs on two register sets so that the bias tiles of the next step
-    // travel while the current one is computed, without register copies.
     const int nsteps = (p.N + 63) / 64;
-    f32x16 tA0, tA1, tB0, tB1;
-    load_btile(0, tA0);
-    load_btile(1, tA1);
-    for (int step = 0; step < nsteps; step += 2) {
+    f32x16 c0, c1;
+    load_btile(0, c0);
+    load_btile(1, c1);
+    for (int step = 0; step < nsteps; ++step) {
         if (step % SPS == 0) stage(step * 64);
-        load_btile(2 * step + 2, tB0);
-        load_btile(2 * step + 3, tB1);
-        if (active) compute(step, tA0, tA1);
-        if (step + 1 < nsteps) {
-            load_btile(2 * step + 4, tA0);
-            load_btile(2 * step + 5, tA1);
-            if (active) compute(step + 1, tB0, tB1);
-        }
+        if (active) compute(step, c0, c1);
     }
 
     if (active) {
@@ -252,17 +248,26 @@ __global__ void __launch_bounds__(256) mfma_fwd(EvoAttnParams p, Extra e) {
     }
 }
 
-template <typename T, int D>
+template <typename T, int D, int NW>
 static int fwd_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const unsigned nqb = (p.N + 127) / 128, grid = nqb * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, false><<<grid, 256, 0, st>>>(p, e);
-    else mfma_fwd<T, D, true><<<grid, 256, 0, st>>>(p, e);
+    const unsigned nqb = (p.N + NW * 32 - 1) / (NW * 32), grid = nqb * (unsigned)(p.B * p.H * p.S);
+    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, false, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    else mfma_fwd<T, D, true, NW><<<grid, NW * 64, 0, st>>>(p, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }
 
+// 8 waves (256 query rows) per workgroup stage K and V once for twice the rows; worth it
+// unless the last workgroup of a problem would be more than half empty.
+template <typename T, int D>
+static int fwd_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    const int rem = p.N % 256;
+    const bool wide = p.N >= 256 && (rem == 0 || rem > 128);
+    return wide ? fwd_bias<T, D, 8>(p, e, st) : fwd_bias<T, D, 4>(p, e, st);
+}
+
 int EVO_CAT(launch_mfma_fwd_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    return p.dtype == EVO_BF16 ? fwd_bias<bf16_t, EVO_D>(p, e, st) : fwd_bias<f16_t, EVO_D>(p, e, st);
+    return p.dtype == EVO_BF16 ? fwd_waves<bf16_t, EVO_D>(p, e, st) : fwd_waves<f16_t, EVO_D>(p, e, st);
 }
 
 }  // namespace evo
