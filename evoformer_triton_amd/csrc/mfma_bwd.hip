@@ -335,16 +335,18 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ dK, dV (and dMask partials)
 //
-// Workgroup = 4 waves = 128 keys of one problem; each wave keeps its 32 keys' K and V
+// Workgroup = NW (4 or 8) waves = NW*32 keys of one problem; each wave keeps its 32 keys' K and V
 // operands in registers and loops over all query rows, staged through LDS both row-major
 // (for S = Q K^T, dP = dO V^T) and transposed (for dV^T += dO^T P, dK^T += Q^T dS).
 // Scores are NOT transposed here: a lane owns one key and 16 queries, so that P and dS in
 // accumulator layout are the B operands of the two gradient matmuls.
-template <typename T, int D, bool HAS_BIAS>
-__global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
+template <typename T, int D, bool HAS_BIAS, int NW>
+__global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     constexpr int KW = G::KW, KS = G::KS, KSD = G::KSD, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
-    constexpr int BK = 128;
+    constexpr int NTH = NW * 64;
+    constexpr int BK = NW * 32;
+    constexpr bool PREFETCH = NW == 4;       // the 8-wave form runs at 128 registers, 4 waves per SIMD
     constexpr int BQS = D <= 32 ? 128 : 64;  // query rows staged per round
     constexpr int TPS = BQS / 32;            // query tiles per stage
     constexpr int RW = G::RESID ? KSD * 16 : 0;  // residue columns of the scaled Q rows
@@ -380,14 +382,14 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
 
     // LDS that is read but never staged
     if (!G::AUG_IN_PAD)
-        for (int r = tid; r < BQS; r += 256) {
+        for (int r = tid; r < BQS; r += NTH) {
             *reinterpret_cast<v8 *>(&Qs[r * QP + AUGC + 8]) = zero8<T>();
             *reinterpret_cast<v8 *>(&Gs[r * QP + AUGC + 8]) = zero8<T>();
         }
     if (G::RESID && D < 16)
-        for (int r = tid; r < BQS; r += 256) *reinterpret_cast<v8 *>(&Qs[r * QP + KW + 8]) = zero8<T>();
+        for (int r = tid; r < BQS; r += NTH) *reinterpret_cast<v8 *>(&Qs[r * QP + KW + 8]) = zero8<T>();
     if (DP > D)
-        for (int i = tid; i < (DP - D) * TP / 8; i += 256) {
+        for (int i = tid; i < (DP - D) * TP / 8; i += NTH) {
             *reinterpret_cast<v8 *>(&Qt[D * TP + i * 8]) = zero8<T>();
             *reinterpret_cast<v8 *>(&Gt[D * TP + i * 8]) = zero8<T>();
         }
@@ -437,7 +439,7 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
 
     auto stage = [&](int qs0) {
         __syncthreads();
-        for (int it = tid; it < BQS * (D / 8); it += 256) {
+        for (int it = tid; it < BQS * (D / 8); it += NTH) {
             const int row = it / (D / 8), ch = it % (D / 8), qq = qs0 + row;
             v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + ch * 8) : zero8<T>();
             v8 bb2 = qq < p.N ? ld8(Gd + (int64_t)qq * sn + ch * 8) : zero8<T>();
@@ -448,7 +450,7 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
             if (G::RESID) *reinterpret_cast<v8 *>(&Qs[row * QP + KW + ch * 8]) = lo;
             *reinterpret_cast<v8 *>(&Gs[row * QP + ch * 8]) = bb2;
         }
-        for (int row = tid; row < BQS; row += 256) {
+        for (int row = tid; row < BQS; row += NTH) {
             const int qq = qs0 + row;
             // rows past N get -LSE = floor: their probabilities vanish
             const float nl = qq < p.N ? -p.lse[pr.row0 + qq] * kLog2e : kMaskFloor;
@@ -457,7 +459,7 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
             *reinterpret_cast<v8 *>(&Gs[row * QP + AUGC]) = aug8<T>(pack_split3<T>(nd), zero3);
         }
         constexpr int NPAIR = BQS / 2;
-        for (int it = tid; it < NPAIR * (D / 8); it += 256) {
+        for (int it = tid; it < NPAIR * (D / 8); it += NTH) {
             const int ch = it / NPAIR, jp = it % NPAIR, r0 = qs0 + 2 * jp;
             v8 qa = r0 < p.N ? ld8(Q + (int64_t)r0 * sn + ch * 8) : zero8<T>();
             v8 qb = r0 + 1 < p.N ? ld8(Q + (int64_t)(r0 + 1) * sn + ch * 8) : zero8<T>();
@@ -477,7 +479,7 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
     };
 
     // one 32-query tile against this wave's 32 keys
-    auto compute = [&](int qtile, const f32x16 &ctile) {
+    auto compute = [&](int qtile, f32x16 &ctile) {
         const int qb = (qtile % TPS) * 32;
         f32x16 acc, dp;
 #pragma unroll
@@ -500,6 +502,8 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
             }
             dp = Mfma<T>::mma(ga, vf[ks], dp);                 // dP - delta
         }
+        // consumed above; with registers to spare the next tile travels during the rest
+        if (PREFETCH) load_btile(qtile + 1, ctile);
         if (G::RESID) {
 #pragma unroll
             for (int ks = 0; ks < KSD; ++ks) {
@@ -539,17 +543,12 @@ __global__ void __launch_bounds__(256) mfma_dkdv(EvoAttnParams p, Extra e) {
         }
     };
 
-    // query tiles in pairs on two register sets (bias tile of the next one in flight)
-    f32x16 tA, tB;
-    load_btile(0, tA);
-    for (int qtile = 0; qtile < NT; qtile += 2) {
+    f32x16 ctile;
+    if (PREFETCH) load_btile(0, ctile);
+    for (int qtile = 0; qtile < NT; ++qtile) {
         if (qtile % TPS == 0) stage(qtile * 32);
-        load_btile(qtile + 1, tB);
-        if (active) compute(qtile, tA);
-        if (qtile + 1 < NT) {
-            load_btile(qtile + 2, tA);
-            if (active) compute(qtile + 1, tB);
-        }
+        if (!PREFETCH) load_btile(qtile, ctile);
+        if (active) compute(qtile, ctile);
     }
 
     if (active) {
@@ -600,12 +599,20 @@ static int dq_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.bias_dtype == EVO_NONE ? dq_ntw<T, D, false>(p, e, st) : dq_ntw<T, D, true>(p, e, st);
 }
 
-template <typename T, int D>
+template <typename T, int D, int NW>
 static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const unsigned grid = (unsigned)((p.N + 127) / 128) * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false><<<grid, 256, 0, st>>>(p, e);
-    else mfma_dkdv<T, D, true><<<grid, 256, 0, st>>>(p, e);
+    const unsigned grid = (unsigned)((p.N + NW * 32 - 1) / (NW * 32)) * (unsigned)(p.B * p.H * p.S);
+    if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    else mfma_dkdv<T, D, true, NW><<<grid, NW * 64, 0, st>>>(p, e);
     return hip_rc();
+}
+
+// 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys; worth it unless
+// the last workgroup of a problem would be more than half empty.
+template <typename T, int D>
+static int dkdv_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    const bool wide = (p.flags & 0x100) != 0;   // measured slower than the 4-wave form at N = 256
+    return wide ? dkdv_bias<T, D, 8>(p, e, st) : dkdv_bias<T, D, 4>(p, e, st);
 }
 
 int EVO_CAT(launch_mfma_dq_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
@@ -613,7 +620,7 @@ int EVO_CAT(launch_mfma_dq_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hip
 }
 
 int EVO_CAT(launch_mfma_dkdv_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    return p.dtype == EVO_BF16 ? dkdv_bias<bf16_t, EVO_D>(p, e, st) : dkdv_bias<f16_t, EVO_D>(p, e, st);
+    return p.dtype == EVO_BF16 ? dkdv_waves<bf16_t, EVO_D>(p, e, st) : dkdv_waves<f16_t, EVO_D>(p, e, st);
 }
 
 }  // namespace evo
