@@ -50,10 +50,10 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def _compile(unit):
+def _compile(unit, extra=(), obj_dir=None):
     name, src, defs = unit
-    out = os.path.join(OBJ, name + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *defs, "-c", os.path.join(CSRC, src), "-o", out]
+    out = os.path.join(obj_dir or OBJ, name + ".o")
+    cmd = [_hipcc(), *HIPCC_FLAGS, *defs, *extra, "-c", os.path.join(CSRC, src), "-o", out]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature" not in l)
     if r.returncode != 0:
@@ -61,28 +61,31 @@ def _compile(unit):
     return out, err
 
 
-def build(force: bool = True, verbose: bool = False, jobs: int | None = None) -> str:
-    """Compile every HIP source for gfx950 and link the shared library."""
-    os.makedirs(OBJ, exist_ok=True)
+def build(force: bool = True, verbose: bool = False, jobs: int | None = None, extra=(), lib_path: str | None = None,
+          obj_dir: str | None = None) -> str:
+    """Compile every HIP source for gfx950 and link the shared library.  `extra` adds compiler
+    flags (e.g. -DEVO_TRACE for a build with phase timestamps) for a library at `lib_path`."""
+    lib_out = lib_path or LIB
+    os.makedirs(obj_dir or OBJ, exist_ok=True)
     units = _units()
-    if not force and os.path.exists(LIB):
+    if not force and not extra and os.path.exists(LIB):
         newest = max(os.path.getmtime(os.path.join(r, f)) for r, _, fs in os.walk(CSRC) for f in fs)
         newest = max(newest, os.path.getmtime(os.path.join(ROOT, "include", "evoattn.h")))
         if os.path.getmtime(LIB) >= newest:
             return LIB
     jobs = jobs or min(8, os.cpu_count() or 1)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        results = list(ex.map(_compile, units))
+        results = list(ex.map(lambda u: _compile(u, extra, obj_dir), units))
     if verbose:
         for _, err in results:
             if err.strip():
                 print(err, file=sys.stderr)
     objs = [o for o, _ in results]
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_out, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
-    return LIB
+    return lib_out
 
 
 if __name__ == "__main__":

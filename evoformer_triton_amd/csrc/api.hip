@@ -145,6 +145,14 @@ static int check_bwd(const EvoAttnParams *p) {
 
 using namespace evo;
 
+#ifdef EVO_TRACE
+static long long *g_trace = nullptr;
+extern "C" void evoattn_set_trace(void *buf) { g_trace = (long long *)buf; }
+#define EVO_SET_TRACE(e) (e).trace = g_trace
+#else
+#define EVO_SET_TRACE(e) do {} while (0)
+#endif
+
 extern "C" {
 
 int evoattn_version(void) { return EVOATTN_VERSION; }
@@ -194,6 +202,7 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     Extra e{};
     e.vec_ok = bias_vec_ok(*p);
     fill_prep(*p, e);
+    EVO_SET_TRACE(e);
     if ((rc = launch_prep(*p, e, st))) return rc;
     return launch_mfma_fwd(*p, e, st);
 }
@@ -215,6 +224,7 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     if (!mfma_ok(*p, EVO_PASS_BWD)) return launch_generic_bwd(*p, e, st);
     if ((rc = check_prep(*p))) return rc;
     fill_prep(*p, e);
+    EVO_SET_TRACE(e);
     if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
     if (p->flags & EVO_FLAG_ONLY_DQ) return launch_mfma_dq(*p, e, st);
     if (p->flags & EVO_FLAG_ONLY_DKDV) return launch_mfma_dkdv(*p, e, st);

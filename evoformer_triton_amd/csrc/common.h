@@ -46,6 +46,7 @@ struct Extra {
     uint2 *m2;         // additive mask * log2(e), shifted, clamped, as (hi, mid, lo, 0) of T  [B][S][NT*32]
     int *dead;         // [B][S] 1 where every key of the row is masked out
     int64_t zero_tile; // offset (floats) of an all-zero tile inside bq and bk
+    long long *trace;  // trace builds only: 16 timestamps per wave
 };
 
 // Linear block id -> logical id such that consecutive logical ids run on one XCD
