@@ -18,6 +18,7 @@ EVO_FLAG_FORCE_GENERIC = 1
 EVO_FLAG_PREP_VALID = 2
 EVO_FLAG_ONLY_DQ = 4
 EVO_FLAG_ONLY_DKDV = 8
+EVO_FLAG_ASYNC_FWD = 16
 EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 

@@ -59,11 +59,20 @@ static int bias_vec_ok(const EvoAttnParams &p) {
     return aligned(p.bias, a) && p.bias_stride_b % 4 == 0 && p.bias_stride_h % 4 == 0 && p.bias_stride_row % 4 == 0;
 }
 
+// The dQ kernel that double-buffers its operands in LDS keeps at most 4 key tiles per wave.
+// Bit 0x200 of flags (not part of the public interface) selects the other form for comparison.
+static bool dq_ring_ok(const EvoAttnParams &p) {
+    return !(p.flags & 0x200) && p.N <= mfma_dqr_max_n(p.D);
+}
+
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
 // writes one partial dBias tile.  Enough chunks to fill the chip, no more.
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
-    const int64_t base = (int64_t)((p.N + 31) / 32) * p.B * p.H;
-    int64_t want = (1024 + base - 1) / base;
+    const int64_t NT = (p.N + 31) / 32;
+    const bool ring = dq_ring_ok(p);   // 64 query rows and 8 waves per workgroup, one workgroup per CU
+    const int64_t base = (ring ? (NT + 1) / 2 : NT) * p.B * p.H;
+    const int64_t target = ring ? 512 : 1024;
+    int64_t want = (target + base - 1) / base;
     if (want < 1) want = 1;
     if (want > p.S) want = p.S;
     *chunk = (int)((p.S + want - 1) / want);
@@ -71,7 +80,7 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
 }
 
 struct PrepLayout {
-    size_t bq, bk, m2, dead, total;
+    size_t bq, bk, m2, m2a, dead, total;
     int bias_batches;
 };
 
@@ -85,6 +94,7 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
     w.bq = off; off += align_up(tiles);
     w.bk = off; off += align_up(tiles);
     w.m2 = off; off += align_up((size_t)p.B * p.S * NT * 32 * 8);
+    w.m2a = off; off += align_up((size_t)p.B * p.S * ((p.N + 255) / 256 * 256) * 16);
     w.dead = off; off += align_up((size_t)p.B * p.S * 4);
     w.total = off;
     return w;
@@ -97,6 +107,7 @@ static void fill_prep(const EvoAttnParams &p, Extra &e) {
     e.bq = (float *)(base + w.bq);
     e.bk = (float *)(base + w.bk);
     e.m2 = (uint2 *)(base + w.m2);
+    e.m2a = (uint4 *)(base + w.m2a);
     e.dead = (int *)(base + w.dead);
     e.zero_tile = (int64_t)w.bias_batches * p.H * ((p.N + 31) / 32) * ((p.N + 31) / 32) * 1024;
 }
@@ -204,7 +215,7 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     fill_prep(*p, e);
     EVO_SET_TRACE(e);
     if ((rc = launch_prep(*p, e, st))) return rc;
-    return launch_mfma_fwd(*p, e, st);
+    return (p->flags & EVO_FLAG_ASYNC_FWD) ? launch_mfma_fwda(*p, e, st) : launch_mfma_fwd(*p, e, st);
 }
 
 int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
@@ -226,10 +237,11 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     fill_prep(*p, e);
     EVO_SET_TRACE(e);
     if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
-    if (p->flags & EVO_FLAG_ONLY_DQ) return launch_mfma_dq(*p, e, st);
+    const bool ring = dq_ring_ok(*p);
+    if (p->flags & EVO_FLAG_ONLY_DQ) return ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st);
     if (p->flags & EVO_FLAG_ONLY_DKDV) return launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads
-    if ((rc = launch_mfma_dq(*p, e, st))) return rc;
+    if ((rc = ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st))) return rc;
     if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;
     if (p->dbias && (rc = launch_dbias_reduce(*p, e, st))) return rc;
     if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;

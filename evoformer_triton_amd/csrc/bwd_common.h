@@ -1,0 +1,57 @@
+// Pieces shared by the backward matrix-core kernels of one head dim.
+#pragma once
+
+#include "common.h"
+
+namespace evo {
+
+// Geometry shared by the two kernels for head dim D.
+template <int D>
+struct Geo {
+    static constexpr bool AUG_IN_PAD = D == 8;           // extra columns fit the zero padding of k-step 0
+    static constexpr int KW = AUG_IN_PAD ? 16 : D + 16;  // operand row: data, extra columns, zeros
+    static constexpr int KS = KW / 16;
+    static constexpr int KSD = (D + 15) / 16;            // k-steps that hold data
+    static constexpr int AUGC = AUG_IN_PAD ? 8 : D;      // first extra column
+    static constexpr int DT = (D + 31) / 32;
+    static constexpr int DP = DT * 32;
+    // The operand scaled by scale*log2(e) is rounded to 16 bits; for small head dims, where
+    // the matrix core has k-steps to spare, its rounding residue is carried as well, which
+    // makes the scores exact to fp32 (and identical in the forward and both backward kernels).
+    static constexpr bool RESID = D <= 16;
+};
+
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 scaled8(typename Mfma<T>::v8 raw, float c) {
+    typename Mfma<T>::v8 r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = (T)((float)raw[i] * c);
+    return r;
+}
+
+// 8 operand columns [a0 a1 a2 b0 b1 b2 0 0] from two packed (hi, mid, lo, 0) triples.
+template <typename T>
+__device__ __forceinline__ typename Mfma<T>::v8 aug8(uint2 a, uint2 b) {
+    typename Mfma<T>::v4 va = __builtin_bit_cast(typename Mfma<T>::v4, a);
+    typename Mfma<T>::v4 vb = __builtin_bit_cast(typename Mfma<T>::v4, b);
+    typename Mfma<T>::v8 r;
+    r[0] = va[0]; r[1] = va[1]; r[2] = va[2];
+    r[3] = vb[0]; r[4] = vb[1]; r[5] = vb[2];
+    r[6] = (T)0.0f; r[7] = (T)0.0f;
+    return r;
+}
+
+template <typename T>
+__device__ __forceinline__ uint2 ones3() {
+    typename Mfma<T>::v4 v;
+    v[0] = v[1] = v[2] = (T)1.0f;
+    v[3] = (T)0.0f;
+    return __builtin_bit_cast(uint2, v);
+}
+
+static inline int hip_rc() {
+    hipError_t err = hipGetLastError();
+    return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
+}
+
+}  // namespace evo

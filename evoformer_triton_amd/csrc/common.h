@@ -44,6 +44,8 @@ struct Extra {
     float *bq;         // bias * log2(e) in accumulator-tile order, lane = query  [Bb][H][NT][NT][64][16]
     float *bk;         // same, lane = key
     uint2 *m2;         // additive mask * log2(e), shifted, clamped, as (hi, mid, lo, 0) of T  [B][S][NT*32]
+    uint4 *m2a;        // the same mask rows as ready-made 16-byte operand chunks (hi, mid, lo, 1, 1, 1, 0, 0),
+                       // padded with the floor to a multiple of 256 keys                        [B][S][NP256]
     int *dead;         // [B][S] 1 where every key of the row is masked out
     int64_t zero_tile; // offset (floats) of an all-zero tile inside bq and bk
     long long *trace;  // trace builds only: 16 timestamps per wave

@@ -6,7 +6,10 @@ namespace evo {
 
 #define EVO_DECL(D)                                                                          \
     int launch_mfma_fwd_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
+    int launch_mfma_fwda_d##D(const EvoAttnParams &, const Extra &, hipStream_t);            \
     int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
+    int launch_mfma_dqr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
+    int mfma_dqr_max_n_d##D();                                                               \
     int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
 EVO_DECL(16)
@@ -25,8 +28,20 @@ EVO_DECL(64)
         return EVO_EUNSUPPORTED;                                              \
     }
 EVO_ROUTE(fwd)
+EVO_ROUTE(fwda)
 EVO_ROUTE(dq)
+EVO_ROUTE(dqr)
 EVO_ROUTE(dkdv)
 #undef EVO_ROUTE
+
+int mfma_dqr_max_n(int D) {
+    switch (D) {
+        case 8: return mfma_dqr_max_n_d8();
+        case 16: return mfma_dqr_max_n_d16();
+        case 32: return mfma_dqr_max_n_d32();
+        case 64: return mfma_dqr_max_n_d64();
+    }
+    return 0;
+}
 
 }  // namespace evo

@@ -22,7 +22,7 @@
 // accumulators (an identity-matrix MFMA adds the dS tile, rounded to fp16 for this purpose:
 // 11 significant bits per term, fp32 sum), writes one partial per chunk, and a second
 // kernel adds the partials in a fixed order: no floating-point atomics, bit-reproducible.
-#include "common.h"
+#include "bwd_common.h"
 #include "kernels.h"
 
 #ifndef EVO_D
@@ -30,50 +30,6 @@
 #endif
 
 namespace evo {
-
-// Geometry shared by the two kernels for head dim D.
-template <int D>
-struct Geo {
-    static constexpr bool AUG_IN_PAD = D == 8;           // extra columns fit the zero padding of k-step 0
-    static constexpr int KW = AUG_IN_PAD ? 16 : D + 16;  // operand row: data, extra columns, zeros
-    static constexpr int KS = KW / 16;
-    static constexpr int KSD = (D + 15) / 16;            // k-steps that hold data
-    static constexpr int AUGC = AUG_IN_PAD ? 8 : D;      // first extra column
-    static constexpr int DT = (D + 31) / 32;
-    static constexpr int DP = DT * 32;
-    // The operand scaled by scale*log2(e) is rounded to 16 bits; for small head dims, where
-    // the matrix core has k-steps to spare, its rounding residue is carried as well, which
-    // makes the scores exact to fp32 (and identical in the forward and both backward kernels).
-    static constexpr bool RESID = D <= 16;
-};
-
-template <typename T>
-__device__ __forceinline__ typename Mfma<T>::v8 scaled8(typename Mfma<T>::v8 raw, float c) {
-    typename Mfma<T>::v8 r;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = (T)((float)raw[i] * c);
-    return r;
-}
-
-// 8 operand columns [a0 a1 a2 b0 b1 b2 0 0] from two packed (hi, mid, lo, 0) triples.
-template <typename T>
-__device__ __forceinline__ typename Mfma<T>::v8 aug8(uint2 a, uint2 b) {
-    typename Mfma<T>::v4 va = __builtin_bit_cast(typename Mfma<T>::v4, a);
-    typename Mfma<T>::v4 vb = __builtin_bit_cast(typename Mfma<T>::v4, b);
-    typename Mfma<T>::v8 r;
-    r[0] = va[0]; r[1] = va[1]; r[2] = va[2];
-    r[3] = vb[0]; r[4] = vb[1]; r[5] = vb[2];
-    r[6] = (T)0.0f; r[7] = (T)0.0f;
-    return r;
-}
-
-template <typename T>
-__device__ __forceinline__ uint2 ones3() {
-    typename Mfma<T>::v4 v;
-    v[0] = v[1] = v[2] = (T)1.0f;
-    v[3] = (T)0.0f;
-    return __builtin_bit_cast(uint2, v);
-}
 
 // ------------------------------------------------------------------ dQ, delta and dBias partials
 //
@@ -575,11 +531,6 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
 }
 
 // ------------------------------------------------------------------ launchers
-
-static inline int hip_rc() {
-    hipError_t err = hipGetLastError();
-    return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
-}
 
 template <typename T, int D, bool HAS_BIAS>
 static int dq_ntw(const EvoAttnParams &p, const Extra &e, hipStream_t st) {

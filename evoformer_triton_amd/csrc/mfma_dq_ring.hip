@@ -1,0 +1,453 @@
+// dQ, delta and dBias partials with the operands of each S row double-buffered in LDS.
+// Compiled once per head dim (-DEVO_D=8|16|32|64).
+//
+// Same arithmetic as `mfma_dq` in mfma_bwd.hip (the reference's `_attn_bwd_preprocess` and
+// `_attn_bwd_dq`, evoformer.py:299-476) and the same ownership: a workgroup keeps a slab of
+// query rows of one head for a whole chunk of S rows, so that the running sum of dS for
+// that slab (the dBias partial) and the slab's bias tiles stay in registers.  What differs
+// is how the per-row operands arrive.  There, every S row starts with loads whose latency
+// nothing hides (a few microseconds, several times the arithmetic of the row).  Here
+//   * the workgroup has 8 waves and a slab of 64 query rows: wave w works on query tile
+//     w / 4 and, of every block of keys, on the 32-key tiles (w % 4), (w % 4) + 4, ...;
+//   * K, V, the mask columns, and the slab's Q, dO and O rows of S row s+1 are requested
+//     (16 bytes per lane and load, 6 loads per wave at D = 32) before row s is computed out
+//     of one LDS buffer, and written to the other buffer when that arithmetic is done; rows
+//     with more keys than one buffer holds go through it in blocks;
+//   * K^T fragments for dQ^T += K^T dS^T come from row-major K by transposing LDS reads
+//     (`ds_read_b64_tr_b16`), so no transposed copy is written.
+// Staging through registers rather than with direct-to-LDS loads is deliberate: measured
+// here, `global_load_lds_dwordx4` moves about 16 bytes per clock and CU and holds up the
+// other waves' LDS reads while it does, a microsecond per S row; a 16-byte `ds_write` per
+// lane does not.
+#include "bwd_common.h"
+#include "kernels.h"
+
+#ifndef EVO_D
+#error "compile with -DEVO_D=<head dim>"
+#endif
+
+namespace evo {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+template <int D>
+struct RingGeo {
+    static constexpr int C = D / 8;                          // 16-byte chunks per row
+    static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
+    static constexpr int BKV = D <= 32 ? 256 : 128;          // keys per stage
+    static constexpr int TPB = BKV / 32;                     // key tiles per stage
+    static constexpr int TPW = TPB / 4;                      // key tiles per stage and wave
+    static constexpr int QR = 64;                            // query rows per workgroup
+    static constexpr int DP = (D + 31) / 32 * 32;
+    static constexpr int RP = DP + 4;                        // pitch of a partial dQ row (floats)
+    static constexpr int K_BYTES = BKV * D * 2;
+    static constexpr int A_BYTES = BKV * 16;
+    static constexpr int Q_BYTES = QR * D * 2;
+    static constexpr int OFF_V = K_BYTES;
+    static constexpr int OFF_A = 2 * K_BYTES;
+    static constexpr int OFF_Q = OFF_A + A_BYTES;
+    static constexpr int OFF_G = OFF_Q + Q_BYTES;
+    static constexpr int OFF_O = OFF_G + Q_BYTES;
+    static constexpr int STAGE_BYTES = OFF_O + Q_BYTES;
+    static constexpr int RED_BYTES = 8 * 32 * RP * 4;
+    static constexpr int BUF_BYTES = ((STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES) + 1023) / 1024 * 1024;
+    static constexpr int LDS_BYTES = 2 * BUF_BYTES;
+    // 1 KB pieces (64 lanes x 16 bytes) per segment of a stage
+    static constexpr int I_K = K_BYTES / 1024, I_A = A_BYTES / 1024, I_Q = Q_BYTES / 1024;
+    static constexpr int I_KVA = 2 * I_K + I_A;
+    static constexpr int I_ALL = I_KVA + 3 * I_Q;
+    // byte offset of chunk c of row r inside a swizzled row-major block
+    static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
+};
+
+// Workgroup barrier that orders LDS traffic only: the loads of the next stage and the stores
+// of the last row stay in flight across it (__syncthreads() would wait for them).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+#ifdef EVO_TRACE
+#define EVO_TR(slot)                                                                             \
+    do {                                                                                         \
+        if (e.trace && (threadIdx.x & 63) == 0 && s == s_begin + 3)                              \
+            e.trace[((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define EVO_TR(slot) do {} while (0)
+#endif
+
+template <typename T, int D, bool HAS_BIAS, int NBLK>
+__global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
+    typedef Geo<D> G;
+    typedef RingGeo<D> R;
+    constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
+    constexpr int C = R::C, BKV = R::BKV, TPB = R::TPB, TPW = R::TPW, RP = R::RP;
+    constexpr int NSLOT = NBLK * TPW;   // key tiles per wave over a whole row
+    typedef typename Mfma<T>::v8 v8;
+    typedef typename Mfma<T>::v4 v4;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar, so that what depends on it branches
+    const int li = lane & 31, g = lane >> 5;
+    const int qi = wave >> 2, kq = wave & 3;
+    const int NT = (p.N + 31) / 32, NQP = (NT + 1) / 2;
+    const int np256 = (p.N + 255) / 256 * 256;
+    const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
+    const int qp = lid % NQP;
+    const unsigned bh = (lid / NQP) % (unsigned)(p.B * p.H);
+    const int c = lid / NQP / (unsigned)(p.B * p.H);
+    const int b = bh / p.H, h = bh % p.H;
+    const int qbase = qp * 64;
+    const int q0 = qbase + qi * 32;
+    const bool qact = q0 < p.N;             // wave-uniform; an odd tile count leaves one pair half empty
+    const int qt = min(q0 >> 5, NT - 1);
+    const int qrow = min(q0 + li, p.N - 1);
+    const int64_t sn = p.stride_n;
+    const bool want_dbias = e.dbias_part != nullptr && p.dbias != nullptr;
+    const float cs = p.scale * kLog2e;
+
+    // identity slices in fp16: A[m][8g+i] = 1 where m is the key row that register 8ts+i of
+    // an accumulator tile holds for lane group g
+    f16x8 idf[2];
+#pragma unroll
+    for (int ts = 0; ts < 2; ++ts)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) idf[ts][i] = (f16_t)(li == crow(8 * ts + i, g) ? 1.0f : 0.0f);
+
+    f32x16 dbacc[NSLOT];
+#pragma unroll
+    for (int j = 0; j < NSLOT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
+
+    // key tile of slot j of this wave
+    auto slot_tile = [&](int j) { return (j / TPW) * TPB + (j % TPW) * 4 + kq; };
+
+    f32x16 bres[HAS_BIAS ? NSLOT : 1];
+    if (HAS_BIAS) {
+        const int bb = e.bias_batches > 1 ? b : 0;
+        const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < NSLOT; ++j) {
+            const float *src = btile0 + (int64_t)min(slot_tile(j), NT - 1) * 1024;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
+                bres[j][4 * rr] = v[0]; bres[j][4 * rr + 1] = v[1]; bres[j][4 * rr + 2] = v[2]; bres[j][4 * rr + 3] = v[3];
+            }
+        }
+    }
+
+    const int s_begin = c * e.chunk, s_end = min(p.S, s_begin + e.chunk);
+    const int T_total = (s_end - s_begin) * NBLK;
+
+    // ---- stage t = (row s_begin + t / NBLK, key block t % NBLK) lives in buffer t & 1.  It is a
+    // list of 1 KB pieces (64 lanes x 16 bytes); piece n belongs to wave n % 8.  Lane i of
+    // piece m of a row-major block fills LDS slot 64 m + i of that block, which the swizzle
+    // assigns to some chunk of some row.
+    constexpr int IPW = (R::I_ALL + 7) / 8;   // most pieces one wave moves per stage
+    u32x4 stg[IPW];
+    // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
+    const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
+    auto piece = [&](int t, int n, const u32x4 *&src, int &dst) {
+        const int s = s_begin + t / NBLK, blk = t % NBLK;
+        if (n >= 2 * R::I_K && n < R::I_KVA) {
+            const int m = n - 2 * R::I_K;
+            src = reinterpret_cast<const u32x4 *>(e.m2a + ((int64_t)b * p.S + s) * np256 + blk * BKV + m * 64 + lane);
+            dst = R::OFF_A + m * 1024;
+        } else {
+            const int64_t pbase = base0 + (int64_t)(s - s_begin) * p.stride_s;
+            const T *base;
+            int m, row0, off;
+            if (n < R::I_K) { base = (const T *)p.k; m = n; row0 = blk * BKV; off = 0; }
+            else if (n < 2 * R::I_K) { base = (const T *)p.v; m = n - R::I_K; row0 = blk * BKV; off = R::OFF_V; }
+            else if (n < R::I_KVA + R::I_Q) { base = (const T *)p.q; m = n - R::I_KVA; row0 = qbase; off = R::OFF_Q; }
+            else if (n < R::I_KVA + 2 * R::I_Q) { base = (const T *)p.dout; m = n - R::I_KVA - R::I_Q; row0 = qbase; off = R::OFF_G; }
+            else { base = (const T *)p.o; m = n - R::I_KVA - 2 * R::I_Q; row0 = qbase; off = R::OFF_O; }
+            const int L = m * 64 + lane;
+            const int r = L / C, cpos = L % C;
+            const int ch = cpos ^ ((r / R::RPB) % C);
+            const int row = min(row0 + r, p.N - 1);
+            src = reinterpret_cast<const u32x4 *>(base + pbase + (int64_t)(row * (int)sn + ch * 8));
+            dst = off + m * 1024;
+        }
+    };
+    // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
+    // the end repeats the last stage) so that the staging registers stay registers.
+    auto fetch = [&](int t) {
+        t = min(t, T_total - 1);
+        const int ninst = (t % NBLK) == 0 ? R::I_ALL : R::I_KVA;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) {
+            const int n = min(wave + 8 * i, ninst - 1);
+            const u32x4 *src;
+            int dst;
+            piece(t, n, src, dst);
+            stg[i] = *src;
+        }
+    };
+    auto stash = [&](int t) {
+        const int ninst = t >= T_total ? 0 : (t % NBLK) == 0 ? R::I_ALL : R::I_KVA;
+        unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) {
+            const int n = wave + 8 * i;
+            if (n < ninst) {
+                const u32x4 *src;
+                int dst;
+                piece(min(t, T_total - 1), n, src, dst);
+                *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
+            }
+        }
+    };
+
+    fetch(0);
+    stash(0);
+    float lse_nxt = 0.0f;
+    if (T_total > 0) lse_nxt = p.lse[(int64_t)(bh * (unsigned)p.S + s_begin) * p.N + qrow];
+
+    const uint2 one3 = ones3<T>();
+    const uint2 zero3 = {0u, 0u};
+    int t = 0;
+    for (int s = s_begin; s < s_end; ++s) {
+        const unsigned pid = bh * (unsigned)p.S + s;
+        Prob pr;
+        pr.b = b; pr.h = h; pr.s = s;
+        pr.base = base0 + (int64_t)(s - s_begin) * p.stride_s;
+        pr.row0 = (int64_t)pid * p.N;
+        const bool dead = e.dead[b * p.S + s] != 0;
+        const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
+
+        v8 qf[KS], gf[KS], qlo[KSD];
+        f32x16 dqacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dqacc[dt][r] = 0.0f;
+        const unsigned char *buf = lds;
+
+#pragma unroll
+        for (int blk = 0; blk < NBLK; ++blk, ++t) {
+            EVO_TR(0);
+            EVO_TR(1);
+            lds_barrier();   // stage t is in LDS; stage t-1 and the last reduction are done with
+            EVO_TR(2);
+            fetch(t + 1);
+            EVO_TR(3);
+            buf = lds + (t & 1) * R::BUF_BYTES;
+
+            if (blk == 0) {
+                // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
+                const float lse2 = lse_nxt * kLog2e;
+                if (s + 1 < s_end) lse_nxt = p.lse[(int64_t)(pid + 1) * p.N + qrow];
+                float dpart = 0.0f;
+#pragma unroll
+                for (int ks = 0; ks < KSD; ++ks) qlo[ks] = zero8<T>();
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const int d0 = ks * 16 + g * 8;
+                    qf[ks] = zero8<T>();
+                    gf[ks] = zero8<T>();
+                    if (d0 < D) {
+                        const int o = R::swz(qi * 32 + li, 2 * ks + g);
+                        const v8 qraw = *reinterpret_cast<const v8 *>(buf + R::OFF_Q + o);
+                        gf[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_G + o);
+                        const v8 oraw = *reinterpret_cast<const v8 *>(buf + R::OFF_O + o);
+                        if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) dpart = fmaf((float)gf[ks][i], (float)oraw[i], dpart);
+                    }
+                }
+                float dl;
+                {
+                    const unsigned u = __float_as_uint(dpart);
+                    auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                    dl = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+                }
+                if (kq == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    if (ks * 16 + g * 8 == AUGC) {
+                        qf[ks] = aug8<T>(one3, pack_split3<T>(-lse2));   // ones x mask, -lse x ones
+                        gf[ks] = aug8<T>(pack_split3<T>(-dl), zero3);    // -delta x ones
+                    }
+                }
+            }
+
+            EVO_TR(4);
+            if (qact) {
+#pragma unroll
+                for (int jj = 0; jj < TPW; ++jj) {
+                    const int tb = jj * 4 + kq;          // tile inside the stage
+                    const int kt = blk * TPB + tb;
+                    if (kt < NT) {  // wave-uniform
+                        const int slot = blk * TPW + jj;
+                        v8 ka[KS], va[KS];
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            const int d0 = ks * 16 + g * 8;
+                            ka[ks] = zero8<T>();
+                            va[ks] = zero8<T>();
+                            if (d0 < D) {
+                                const int o = R::swz(tb * 32 + li, 2 * ks + g);
+                                ka[ks] = *reinterpret_cast<const v8 *>(buf + o);
+                                va[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_V + o);
+                            } else if (d0 == AUGC) {
+                                ka[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (tb * 32 + li) * 16);  // mask x ones, ones x -lse
+                                va[ks] = aug8<T>(one3, zero3);                                                 // ones x -delta
+                            }
+                        }
+                        f32x16 acc, dp;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[r] = dp[r] = 0.0f;
+                        if (HAS_BIAS && !dead) acc = bres[slot];
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            acc = Mfma<T>::mma(ka[ks], qf[ks], acc);   // log2 P^T
+                            if (G::RESID && ks < KSD) acc = Mfma<T>::mma(ka[ks], qlo[ks], acc);
+                            dp = Mfma<T>::mma(va[ks], gf[ks], dp);     // dP^T - delta
+                        }
+                        float ds[16];
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) ds[r] = kill ? 0.0f : fast_exp2(acc[r]) * dp[r];
+#pragma unroll
+                        for (int ts = 0; ts < 2; ++ts) {
+                            v8 dsf;
+                            f16x8 dsh;
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                dsf[i] = (T)ds[8 * ts + i];
+                                dsh[i] = (f16_t)ds[8 * ts + i];
+                            }
+                            if (want_dbias) dbacc[slot] = Mfma<f16_t>::mma(idf[ts], dsh, dbacc[slot]);
+#pragma unroll
+                            for (int dt = 0; dt < DT; ++dt) {
+                                // K^T fragment: row d = dt*32 + li, the 8 keys the dS^T registers hold
+                                const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                                v8 kta = zero8<T>();
+                                if (col < D) {
+#pragma unroll
+                                    for (int h2 = 0; h2 < 2; ++h2) {
+                                        const int row = tb * 32 + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                                        const unsigned char *ad = buf + R::swz(row, col >> 3) + (col & 7) * 2;
+                                        s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                            (s16x4 __attribute__((address_space(3))) *)ad);
+                                        v4 rv = __builtin_bit_cast(v4, rd);
+                                        kta[4 * h2] = rv[0]; kta[4 * h2 + 1] = rv[1]; kta[4 * h2 + 2] = rv[2]; kta[4 * h2 + 3] = rv[3];
+                                    }
+                                }
+                                dqacc[dt] = Mfma<T>::mma(kta, dsf, dqacc[dt]);
+                            }
+                        }
+                    }
+                }
+            }
+            stash(t + 1);   // into the other buffer, free since the barrier above
+        }
+
+        // Partial dQ^T of this wave: lane = query li, register r = dim dt*32 + crow(r, g).  The
+        // four waves of a query tile meet in the buffer of the stage just consumed.
+        EVO_TR(5);
+        lds_barrier();
+        EVO_TR(6);
+        float *red = (float *)(lds + ((t - 1) & 1) * R::BUF_BYTES);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                f32x4 v;
+                v[0] = dqacc[dt][4 * rr]; v[1] = dqacc[dt][4 * rr + 1];
+                v[2] = dqacc[dt][4 * rr + 2]; v[3] = dqacc[dt][4 * rr + 3];
+                *reinterpret_cast<f32x4 *>(&red[(wave * 32 + li) * RP + dt * 32 + 8 * rr + 4 * g]) = v;
+            }
+        EVO_TR(7);
+        lds_barrier();
+        EVO_TR(8);
+        T *dQ = (T *)p.dq + pr.base;
+        for (int it = tid; it < 64 * (D / 4); it += 512) {
+            const int q = it / (D / 4), d4 = (it % (D / 4)) * 4;
+            const int w0 = (q >> 5) * 4, ql = q & 31;
+            f32x4 sum = *reinterpret_cast<const f32x4 *>(&red[(w0 * 32 + ql) * RP + d4]);
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
+            if (qbase + q < p.N)
+                store4<T>(dQ + (int64_t)(qbase + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
+                          sum[3] * p.scale);
+        }
+        EVO_TR(9);
+        // the barrier at the top of the next stage keeps the next request for this buffer
+        // behind these reads
+    }
+
+    if (want_dbias && qact && q0 + li < p.N) {
+        float *part = e.dbias_part + ((((int64_t)c * p.B + b) * p.H + h) * p.N + (q0 + li)) * p.N;
+        const bool v4ok = (p.N & 3) == 0;
+#pragma unroll
+        for (int j = 0; j < NSLOT; ++j) {
+            const int kb = slot_tile(j) * 32;
+            if (kb < p.N) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int kg = kb + 8 * rr + 4 * g;
+                    if (v4ok && kg + 4 <= p.N) {
+                        f32x4 v;
+                        v[0] = dbacc[j][4 * rr]; v[1] = dbacc[j][4 * rr + 1];
+                        v[2] = dbacc[j][4 * rr + 2]; v[3] = dbacc[j][4 * rr + 3];
+                        *reinterpret_cast<f32x4 *>(part + kg) = v;
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (kg + i < p.N) part[kg + i] = dbacc[j][4 * rr + i];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launcher
+
+template <typename T, int D, bool HAS_BIAS, int NBLK>
+static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    typedef RingGeo<D> R;
+    static bool attr_set = false;
+    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK>;
+    if (!attr_set) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES) != hipSuccess)
+            return EVO_EHIP;
+        attr_set = true;
+    }
+    const int NT = (p.N + 31) / 32, NQP = (NT + 1) / 2;
+    const unsigned grid = (unsigned)NQP * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
+    kern<<<grid, 512, R::LDS_BYTES, st>>>(p, e);
+    return hip_rc();
+}
+
+template <typename T, int D, bool HAS_BIAS>
+static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    typedef RingGeo<D> R;
+    const int nblk = (p.N + R::BKV - 1) / R::BKV;
+    if (nblk * R::TPW > 4) return EVO_EUNSUPPORTED;
+    if (nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1>(p, e, st);
+    if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2>(p, e, st);
+    if constexpr (R::TPW == 1) {
+        if (nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3>(p, e, st);
+        if (nblk == 4) return dqr_launch<T, D, HAS_BIAS, 4>(p, e, st);
+    }
+    return EVO_EUNSUPPORTED;
+}
+
+template <typename T, int D>
+static int dqr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    return p.bias_dtype == EVO_NONE ? dqr_blocks<T, D, false>(p, e, st) : dqr_blocks<T, D, true>(p, e, st);
+}
+
+// Largest N the double-buffered dQ kernel takes for this head dim (4 key tiles per wave).
+int EVO_CAT(mfma_dqr_max_n_d, EVO_D)() { return 4 / RingGeo<EVO_D>::TPW * RingGeo<EVO_D>::BKV; }
+
+int EVO_CAT(launch_mfma_dqr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    return p.dtype == EVO_BF16 ? dqr_bias<bf16_t, EVO_D>(p, e, st) : dqr_bias<f16_t, EVO_D>(p, e, st);
+}
+
+}  // namespace evo

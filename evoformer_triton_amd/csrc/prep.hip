@@ -81,6 +81,16 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
         }
         out[j] = p.dtype == EVO_F16 ? pack_split3<f16_t>(v) : pack_split3<bf16_t>(v);
     }
+    const int np256 = (p.N + 255) / 256 * 256;
+    uint4 *outa = e.m2a + (int64_t)row * np256;
+    const uint2 fl = p.dtype == EVO_F16 ? pack_split3<f16_t>(kMaskFloor) : pack_split3<bf16_t>(kMaskFloor);
+    // (hi, mid, lo, 1, 1, 1, 0, 0): the ones meet the -LSE columns of the backward's score
+    // MFMA; the forward multiplies them by zeros
+    const unsigned one = p.dtype == EVO_F16 ? 0x3C00u : 0x3F80u;
+    for (int j = tid; j < np256; j += 256) {
+        const uint2 v = j < npad ? out[j] : fl;
+        outa[j] = make_uint4(v.x, v.y | (one << 16), one | (one << 16), 0u);
+    }
     if (tid == 0) e.dead[row] = dead ? 1 : 0;
 }
 

@@ -59,7 +59,8 @@ enum {
      * the dQ kernel (dq, delta and the dBias partials, no final dBias sum); ONLY_DKDV runs
      * the dK/dV kernel and needs the delta a previous full call left in the same workspace. */
     EVO_FLAG_ONLY_DQ       = 4,
-    EVO_FLAG_ONLY_DKDV     = 8
+    EVO_FLAG_ONLY_DKDV     = 8,
+    EVO_FLAG_ASYNC_FWD     = 16 /* forward: the persistent, asynchronously staged kernel */
 };
 
 /* error codes */
