@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device-to-device copy three times: under rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
     return ap.parse_args()
 
 
@@ -150,7 +153,16 @@ def main():
     t_abi = timed(lambda: (call(lib.evoattn_fwd, 0), call(lib.evoattn_bwd, V)), n_k)
     dom = max(t_phase, key=t_phase.get)
     achieved = phases[dom][1] / t_phase[dom] / 1e12
-    kernel_names = {"fwd": "mfma_fwd", "bwd_dq": "mfma_dq", "bwd_dkdv": "mfma_dkdv"}
+    p.flags = 0
+    k_fwd = lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_FWD).decode()
+    k_dq, k_dkdv = lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().split(",")
+    kernel_names = {"fwd": "prep_kernel+" + k_fwd, "bwd_dq": k_dq, "bwd_dkdv": k_dkdv}
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     esz = qc.element_size()
     io_bytes = 12 * qc.numel() * esz + 2 * bias.numel() * bias.element_size()   # algorithmic HBM bytes per step

@@ -18,12 +18,12 @@ EVO_FLAG_FORCE_GENERIC = 1
 EVO_FLAG_PREP_VALID = 2
 EVO_FLAG_ONLY_DQ = 4
 EVO_FLAG_ONLY_DKDV = 8
-EVO_FLAG_ASYNC_FWD = 16
+EVO_FLAG_PER_PROBLEM = 16
 EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 
 EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_prep_bytes", "evoattn_bwd_workspace_bytes",
-           "evoattn_fwd", "evoattn_bwd", "evoattn_path")
+           "evoattn_fwd", "evoattn_bwd", "evoattn_path", "evoattn_kernels")
 
 
 class EvoAttnParams(ctypes.Structure):
@@ -83,7 +83,9 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_bwd.restype = ctypes.c_int
     lib.evoattn_bwd.argtypes = [P, ctypes.c_void_p]
     lib.evoattn_path.restype = ctypes.c_char_p
+    lib.evoattn_kernels.restype = ctypes.c_char_p
     lib.evoattn_path.argtypes = [P, ctypes.c_int]
+    lib.evoattn_kernels.argtypes = [P, ctypes.c_int]
     _LIB = lib
     return lib
 

@@ -40,7 +40,7 @@ def _units():
     for d in HEAD_DIMS:
         units.append((f"mfma_fwd_d{d}", "mfma_fwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_bwd_d{d}", "mfma_bwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
-        units.append((f"mfma_fwda_d{d}", "mfma_fwd_async.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
+        units.append((f"mfma_fwdr_d{d}", "mfma_fwd_ring.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_dqr_d{d}", "mfma_dq_ring.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
     return units
 

@@ -60,9 +60,8 @@ static int bias_vec_ok(const EvoAttnParams &p) {
 }
 
 // The dQ kernel that double-buffers its operands in LDS keeps at most 4 key tiles per wave.
-// Bit 0x200 of flags (not part of the public interface) selects the other form for comparison.
 static bool dq_ring_ok(const EvoAttnParams &p) {
-    return !(p.flags & 0x200) && p.N <= mfma_dqr_max_n(p.D);
+    return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N <= mfma_dqr_max_n(p.D);
 }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
@@ -204,6 +203,18 @@ const char *evoattn_path(const EvoAttnParams *p, int pass) {
     return mfma_ok(*p, pass) ? "mfma" : "generic";
 }
 
+// rows of 129..256 keys: a workgroup per chunk of S rows with the bias tiles resident
+static bool fwd_ring_ok(const EvoAttnParams &p) {
+    return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
+}
+
+const char *evoattn_kernels(const EvoAttnParams *p, int pass) {
+    if (!p) return "invalid";
+    if (!mfma_ok(*p, pass)) return "generic";
+    if (pass == EVO_PASS_FWD) return fwd_ring_ok(*p) ? "mfma_fwd_ring" : "mfma_fwd";
+    return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv" : "mfma_dq,mfma_dkdv";
+}
+
 int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     int rc = evoattn_check(p, EVO_PASS_FWD);
     if (rc) return rc;
@@ -215,7 +226,8 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     fill_prep(*p, e);
     EVO_SET_TRACE(e);
     if ((rc = launch_prep(*p, e, st))) return rc;
-    return (p->flags & EVO_FLAG_ASYNC_FWD) ? launch_mfma_fwda(*p, e, st) : launch_mfma_fwd(*p, e, st);
+    if (fwd_ring_ok(*p)) return launch_mfma_fwdr(*p, e, st);
+    return launch_mfma_fwd(*p, e, st);
 }
 
 int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {

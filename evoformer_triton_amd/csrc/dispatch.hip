@@ -6,7 +6,8 @@ namespace evo {
 
 #define EVO_DECL(D)                                                                          \
     int launch_mfma_fwd_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
-    int launch_mfma_fwda_d##D(const EvoAttnParams &, const Extra &, hipStream_t);            \
+    int launch_mfma_fwdr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);            \
+    int mfma_fwdr_max_n_d##D();                                                              \
     int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
     int launch_mfma_dqr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
     int mfma_dqr_max_n_d##D();                                                               \
@@ -28,11 +29,21 @@ EVO_DECL(64)
         return EVO_EUNSUPPORTED;                                              \
     }
 EVO_ROUTE(fwd)
-EVO_ROUTE(fwda)
+EVO_ROUTE(fwdr)
 EVO_ROUTE(dq)
 EVO_ROUTE(dqr)
 EVO_ROUTE(dkdv)
 #undef EVO_ROUTE
+
+int mfma_fwdr_max_n(int D) {
+    switch (D) {
+        case 8: return mfma_fwdr_max_n_d8();
+        case 16: return mfma_fwdr_max_n_d16();
+        case 32: return mfma_fwdr_max_n_d32();
+        case 64: return mfma_fwdr_max_n_d64();
+    }
+    return 0;
+}
 
 int mfma_dqr_max_n(int D) {
     switch (D) {

@@ -15,7 +15,8 @@ int launch_mask_shift(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 
 int launch_prep(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_fwd(const EvoAttnParams &p, const Extra &e, hipStream_t st);
-int launch_mfma_fwda(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int launch_mfma_fwdr(const EvoAttnParams &p, const Extra &e, hipStream_t st);
+int mfma_fwdr_max_n(int D);  // largest N the chunk-of-rows forward takes, 0 for a head dim it is not built for
 int launch_mfma_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_dqr(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int mfma_dqr_max_n(int D);  // largest N the double-buffered dQ kernel takes, 0 for an unknown head dim

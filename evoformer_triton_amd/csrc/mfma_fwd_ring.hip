@@ -1,0 +1,369 @@
+// Forward for rows of at most 256 keys: one workgroup walks over a chunk of S rows of one
+// head with the head's bias tiles resident in registers.  Compiled once per head dim.
+//
+// Same arithmetic as mfma_fwd.hip (the reference's `_attn_fwd`, evoformer.py:23-297).  That
+// kernel is one workgroup per (b, h, s) problem: every problem starts with loads whose
+// latency nothing hides, and every problem reads its N x N bias tiles again (fp32, from L2),
+// which at N = 256, D = 32 is four times the bytes of Q, K, V and O together.  Here
+//   * a workgroup has 8 waves = 256 query rows (all of them) and a fixed head; wave w keeps
+//     the bias tiles (query tile w) x (key tiles 0..7) in 128 registers for the whole chunk
+//     of S rows, so the bias is read once per chunk instead of once per row;
+//   * K, V and the mask columns of row s+1 are requested (16 bytes per lane and load) before
+//     row s is computed out of one LDS buffer and written into the other one afterwards; a
+//     wave's own Q rows are prefetched straight into its registers;
+//   * V^T fragments come from row-major V by transposing LDS reads (`ds_read_b64_tr_b16`);
+//   * one workgroup barrier per S row.
+// K and V rows sit in LDS row-major without padding; 16-byte chunks are XOR-swizzled by row
+// so that the operand reads and the transposing reads are free of bank conflicts.
+#include "common.h"
+#include "kernels.h"
+
+#ifndef EVO_D
+#error "compile with -DEVO_D=<head dim>"
+#endif
+
+namespace evo {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+template <int D>
+struct FwdRingGeo {
+    static constexpr int C = D / 8;                          // 16-byte chunks per row
+    static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
+    static constexpr int BKV = 256;                          // keys per stage = most keys per row
+    static constexpr int K_BYTES = BKV * D * 2;
+    static constexpr int A_BYTES = BKV * 16;
+    static constexpr int OFF_V = K_BYTES;
+    static constexpr int OFF_A = 2 * K_BYTES;
+    static constexpr int BUF_BYTES = 2 * K_BYTES + A_BYTES;
+    static constexpr int LDS_BYTES = 2 * BUF_BYTES;
+    // 1 KB pieces (64 lanes x 16 bytes) per segment of a stage
+    static constexpr int I_K = K_BYTES / 1024, I_A = A_BYTES / 1024;
+    static constexpr int I_ALL = 2 * I_K + I_A;
+    static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
+};
+
+// Workgroup barrier that orders LDS traffic only: the loads of the next row and the stores
+// of the last one stay in flight across it (__syncthreads() would wait for them).
+__device__ __forceinline__ void lds_barrier_f() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <typename T, int D, bool HAS_BIAS>
+__global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
+    typedef FwdRingGeo<D> R;
+    constexpr int C = R::C;
+    constexpr int KSD = (D + 15) / 16;             // data k-steps
+    constexpr bool AUG_IN_PAD = D == 8;            // mask columns share k-step 0 with the data
+    constexpr int KS = AUG_IN_PAD ? 1 : KSD + 1;
+    constexpr int DT = (D + 31) / 32;
+    constexpr bool RESID = D <= 16;
+    constexpr float TAU = 8.0f;
+    constexpr int IPW = (R::I_ALL + 7) / 8;        // most pieces one wave moves per stage
+    typedef typename Mfma<T>::v8 v8;
+    typedef typename Mfma<T>::v4 v4;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, g = lane >> 5;
+    const int NT = (p.N + 31) / 32;
+    const int np256 = (p.N + 255) / 256 * 256;
+    const int nsteps = (p.N + 63) / 64;
+    const unsigned bh = blockIdx.x % (unsigned)(p.B * p.H);
+    const int c = blockIdx.x / (unsigned)(p.B * p.H);
+    const int b = bh / p.H, h = bh % p.H;
+    const int q0 = wave * 32;
+    const bool qact = q0 < p.N;
+    const int qrow = min(q0 + li, p.N - 1);
+    const int64_t sn = p.stride_n;
+    const float cscale = p.scale * kLog2e;
+
+    f32x16 bres[HAS_BIAS ? 8 : 1];
+    if (HAS_BIAS) {
+        const int bb = e.bias_batches > 1 ? b : 0;
+        const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + min(wave, NT - 1)) * NT) * 1024 + lane * 16;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float *src = btile0 + (int64_t)min(j, NT - 1) * 1024;
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
+                bres[j][4 * rr] = v[0]; bres[j][4 * rr + 1] = v[1]; bres[j][4 * rr + 2] = v[2]; bres[j][4 * rr + 3] = v[3];
+            }
+        }
+    }
+
+    const int s_begin = c * e.chunk, s_end = min(p.S, s_begin + e.chunk);
+    const int nrows = s_end - s_begin;
+    if (nrows <= 0) return;   // uniform over the workgroup
+    // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
+    const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
+
+    // ---- the stage of row s_begin + t lives in buffer t & 1.  It is a list of 1 KB pieces
+    // (64 lanes x 16 bytes); piece n belongs to wave n % 8.  Lane i of piece m of K or V fills
+    // LDS slot 64 m + i of that block, which the swizzle assigns to some chunk of some row.
+    u32x4 stg[IPW];
+    auto piece = [&](int t, int n, const u32x4 *&src, int &dst) {
+        if (n >= 2 * R::I_K) {
+            const int m = n - 2 * R::I_K;
+            src = reinterpret_cast<const u32x4 *>(e.m2a + ((int64_t)b * p.S + s_begin + t) * np256 + m * 64 + lane);
+            dst = R::OFF_A + m * 1024;
+        } else {
+            const bool isv = n >= R::I_K;
+            const int m = isv ? n - R::I_K : n;
+            const T *base = isv ? (const T *)p.v : (const T *)p.k;
+            const int L = m * 64 + lane;
+            const int r = L / C, cpos = L % C;
+            const int ch = cpos ^ ((r / R::RPB) % C);
+            const int row = min(r, p.N - 1);
+            src = reinterpret_cast<const u32x4 *>(base + base0 + (int64_t)t * p.stride_s + (int64_t)(row * (int)sn + ch * 8));
+            dst = (isv ? R::OFF_V : 0) + m * 1024;
+        }
+    };
+    // Loads are unconditional (a wave with fewer pieces repeats its last one, the row past the
+    // end repeats the last row) so that the staging registers stay registers.
+    auto fetch = [&](int t) {
+        t = min(t, nrows - 1);
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) {
+            const int n = min(wave + 8 * i, R::I_ALL - 1);
+            const u32x4 *src;
+            int dst;
+            piece(t, n, src, dst);
+            stg[i] = *src;
+        }
+    };
+    auto stash = [&](int t) {
+        if (t >= nrows) return;
+        unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) {
+            const int n = wave + 8 * i;
+            if (n < R::I_ALL) {
+                const u32x4 *src;
+                int dst;
+                piece(t, n, src, dst);
+                *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
+            }
+        }
+    };
+    // this lane's half of its query row, straight from global memory
+    v8 qraw[KSD], qnext[KSD];
+    auto fetch_q = [&](int t, v8 (&dst)[KSD]) {
+        t = min(t, nrows - 1);
+        const T *Q = (const T *)p.q + base0 + (int64_t)t * p.stride_s + (int64_t)qrow * sn;
+#pragma unroll
+        for (int ks = 0; ks < KSD; ++ks) {
+            const int ch = 2 * ks + g;
+            dst[ks] = ld8(Q + (ch < C ? ch : 0) * 8);
+        }
+    };
+
+    fetch(0);
+    fetch_q(0, qraw);
+    stash(0);
+
+    for (int t = 0; t < nrows; ++t) {
+        const int s = s_begin + t;
+        const unsigned pid = bh * (unsigned)p.S + s;
+        const bool dead = e.dead[b * p.S + s] != 0;
+        lds_barrier_f();   // the stage of this row is in LDS; everybody is done with the row before
+        fetch(t + 1);
+        fetch_q(t + 1, qnext);
+        const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+
+        if (qact) {
+            v8 qf[KSD], qlo[KSD];
+            const float cq = dead ? 0.0f : cscale;
+#pragma unroll
+            for (int ks = 0; ks < KSD; ++ks) {
+                qf[ks] = zero8<T>();
+                qlo[ks] = zero8<T>();
+                if (2 * ks + g < C) scaled_hilo8<T>(qraw[ks], cq, qf[ks], qlo[ks]);
+            }
+            float m = -INFINITY, l = 0.0f;
+            f32x16 oacc[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
+
+#pragma unroll
+            for (int step = 0; step < 4; ++step) {
+                if (step < nsteps) {  // uniform
+                    const int kb = step * 64;
+                    // ---- scores: S^T = K Q^T (+ bias tiles as C, + mask columns)
+                    f32x16 a0, a1;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        v8 k0, k1, qb;
+                        if (ks < KSD) {
+                            const int ch = 2 * ks + g;
+                            if (AUG_IN_PAD && g == 1) {
+                                k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
+                                k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
+                                qb = zero8<T>();
+                                qb[0] = qb[1] = qb[2] = (T)1.0f;
+                            } else {
+                                k0 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + li, ch < C ? ch : 0));
+                                k1 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + 32 + li, ch < C ? ch : 0));
+                                qb = qf[ks];
+                            }
+                        } else {  // the mask k-step: columns 0..2 of lane group 0
+                            k0 = zero8<T>();
+                            k1 = zero8<T>();
+                            qb = zero8<T>();
+                            if (g == 0) {
+                                k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
+                                k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
+                                qb[0] = qb[1] = qb[2] = (T)1.0f;
+                            }
+                        }
+                        if (ks == 0) {
+                            f32x16 z;
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                            if (HAS_BIAS && !dead) {  // uniform
+                                a0 = Mfma<T>::mma(k0, qb, bres[2 * step]);
+                                a1 = Mfma<T>::mma(k1, qb, bres[2 * step + 1]);
+                            } else {
+                                a0 = Mfma<T>::mma(k0, qb, z);
+                                a1 = Mfma<T>::mma(k1, qb, z);
+                            }
+                        } else {
+                            a0 = Mfma<T>::mma(k0, qb, a0);
+                            a1 = Mfma<T>::mma(k1, qb, a1);
+                        }
+                        if (RESID && ks < KSD) {
+                            v8 ql = (AUG_IN_PAD && g == 1) ? zero8<T>() : qlo[ks];
+                            a0 = Mfma<T>::mma(k0, ql, a0);
+                            a1 = Mfma<T>::mma(k1, ql, a1);
+                        }
+                    }
+                    // ---- online softmax
+                    float mloc = fmaxf(a0[0], a1[0]);
+#pragma unroll
+                    for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
+                    {   // exchange between the two lane groups without touching LDS
+                        const unsigned u = __float_as_uint(mloc);
+                        auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                        mloc = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                    }
+                    // rescale only when the max grows by more than 2^TAU
+                    const bool grow = mloc > m + TAU;
+                    if (__any(grow)) {
+                        const float mn = grow ? mloc : m;
+                        const float alpha = fast_exp2(m - mn);
+                        l *= alpha;
+                        m = mn;
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+                    }
+                    float psum = 0.0f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        a0[r] = fast_exp2(a0[r] - m);
+                        a1[r] = fast_exp2(a1[r] - m);
+                        psum += a0[r] + a1[r];
+                    }
+                    l += psum;
+                    // ---- O^T += V^T P^T, V^T fragments by transposing reads of row-major V
+#pragma unroll
+                    for (int ts = 0; ts < 4; ++ts) {
+                        v8 pf;
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) {
+                            const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                            v8 va = zero8<T>();
+                            if (col < D) {
+#pragma unroll
+                                for (int h2 = 0; h2 < 2; ++h2) {
+                                    const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                                    const unsigned char *ad = buf + R::OFF_V + R::swz(row, col >> 3) + (col & 7) * 2;
+                                    s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                        (s16x4 __attribute__((address_space(3))) *)ad);
+                                    v4 rv = __builtin_bit_cast(v4, rd);
+                                    va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
+                                }
+                            }
+                            oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
+                        }
+                    }
+                }
+            }
+
+            {   // the two lane groups hold the two halves of each query's sum
+                const unsigned u = __float_as_uint(l);
+                auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                l = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+            }
+            const float inv = 1.0f / l;
+            const int q = q0 + li;
+            if (q < p.N) {
+                T *O = (T *)p.o + base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
+                if (g == 0) p.lse[(int64_t)pid * p.N + q] = (m + __log2f(l)) * kLn2;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int d0 = dt * 32 + 8 * rr + 4 * g;
+                        if (d0 < D)
+                            store4<T>(O + d0, oacc[dt][4 * rr] * inv, oacc[dt][4 * rr + 1] * inv,
+                                      oacc[dt][4 * rr + 2] * inv, oacc[dt][4 * rr + 3] * inv);
+                    }
+            }
+        }
+        stash(t + 1);   // into the other buffer, free since the barrier above
+#pragma unroll
+        for (int ks = 0; ks < KSD; ++ks) qraw[ks] = qnext[ks];
+    }
+}
+
+// ------------------------------------------------------------------ launcher
+
+template <typename T, int D, bool HAS_BIAS>
+static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
+    typedef FwdRingGeo<D> R;
+    static int cus = 0;
+    static bool attr_set = false;
+    auto kern = mfma_fwd_ring<T, D, HAS_BIAS>;
+    if (!attr_set) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        hipError_t err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES);
+        if (err != hipSuccess) return EVO_EHIP - (int)err;
+        attr_set = true;
+    }
+    // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
+    Extra e = e0;
+    const int bh = p.B * p.H;
+    int want = (cus + bh - 1) / bh;
+    if (want < 1) want = 1;
+    if (want > p.S) want = p.S;
+    e.chunk = (p.S + want - 1) / want;
+    e.n_chunks = (p.S + e.chunk - 1) / e.chunk;
+    kern<<<(unsigned)bh * (unsigned)e.n_chunks, 512, R::LDS_BYTES, st>>>(p, e);
+    hipError_t err = hipGetLastError();
+    return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
+}
+
+template <typename T>
+static int fwdr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    return p.bias_dtype == EVO_NONE ? fwdr_launch<T, EVO_D, false>(p, e, st) : fwdr_launch<T, EVO_D, true>(p, e, st);
+}
+
+// Largest N this kernel takes for the head dim (0: not built for it).
+int EVO_CAT(mfma_fwdr_max_n_d, EVO_D)() { return EVO_D <= 32 ? 256 : 0; }   // 64: the resident tiles do not fit the registers
+
+int EVO_CAT(launch_mfma_fwdr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    if (EVO_D > 32) return EVO_EUNSUPPORTED;
+    return p.dtype == EVO_BF16 ? fwdr_bias<bf16_t>(p, e, st) : fwdr_bias<f16_t>(p, e, st);
+}
+
+}  // namespace evo

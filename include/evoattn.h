@@ -60,7 +60,9 @@ enum {
      * the dK/dV kernel and needs the delta a previous full call left in the same workspace. */
     EVO_FLAG_ONLY_DQ       = 4,
     EVO_FLAG_ONLY_DKDV     = 8,
-    EVO_FLAG_ASYNC_FWD     = 16 /* forward: the persistent, asynchronously staged kernel */
+    /* Measurement aid: run the one-workgroup-per-(b,h,s) forms of the forward and dQ kernels
+     * also where the forms that walk over a chunk of S rows apply (same results). */
+    EVO_FLAG_PER_PROBLEM   = 16
 };
 
 /* error codes */
@@ -144,6 +146,10 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream);
 /* Name of the kernel family evoattn_fwd/evoattn_bwd would run for these parameters
  * ("mfma" or "generic"); for tests and reports. */
 const char *evoattn_path(const EvoAttnParams *p, int pass);
+
+/* Names of the main kernels that pass would launch, comma separated (e.g. "mfma_fwd_ring",
+ * "mfma_dq_ring,mfma_dkdv", "generic"); for reports and profiles. */
+const char *evoattn_kernels(const EvoAttnParams *p, int pass);
 
 #ifdef __cplusplus
 }

@@ -177,6 +177,13 @@ SMALL = [
     (1, 1, 1280, 1, 64, "bool", torch.float32, "reference"),
     (1, 4, 128, 2, 32, "add", "q", "ds4sci"),
     (2, 3, 72, 4, 16, "soft", torch.float32, "ds4sci"),
+    # 129..256 residues: the kernels that walk over a chunk of S rows
+    (1, 5, 256, 2, 32, "add", "q", "reference"),
+    (1, 3, 200, 2, 16, "bool", torch.float32, "reference"),
+    (2, 4, 130, 3, 8, "soft", "q", "reference"),
+    (1, 3, 250, 2, 64, "add", "q", "reference"),
+    (1, 40, 256, 1, 32, "add", "q", "ds4sci"),
+    (1, 9, 192, 2, 32, None, None, "reference"),
 ]
 
 
@@ -207,6 +214,28 @@ def test_small_cases_bf16(E, case):
     fmask = m is not None and m.dtype != torch.bool
     got = run_hip(E, Q, K, V, m, bias, dO, layout=layout, mask_grad=fmask)
     assert_close(got, ref, BF16_TOL, ["O", "dQ", "dK", "dV", "dBias"] + (["dMask"] if fmask else []), what=str(case))
+
+
+@pytest.mark.parametrize("shape,mask", [((1, 37, 256, 2, 32), "add"), ((1, 5, 200, 3, 16), "bool"),
+                                        ((2, 3, 130, 2, 8), "soft"), ((1, 4, 384, 2, 32), "add"),
+                                        ((1, 3, 480, 1, 64), "add")])
+def test_chunk_of_rows_kernels_match_per_problem_kernels(E, shape, mask):
+    """The forms that walk over a chunk of S rows and the one-workgroup-per-problem forms do
+    the same arithmetic up to the order of a few fp32 additions: results agree to a
+    bf16 unit in the last place."""
+    from evoformer_triton_amd import _lib
+    B, S, N, H, D = shape
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, "q", torch.bfloat16, seed=3)
+    fmask = m.dtype != torch.bool
+    try:
+        E.FLAGS = _lib.EVO_FLAG_PER_PROBLEM
+        a = run_hip(E, Q, K, V, m, bias, dO, mask_grad=fmask)
+    finally:
+        E.FLAGS = 0
+    b = run_hip(E, Q, K, V, m, bias, dO, mask_grad=fmask)
+    for name in a:
+        tol = 2.0 ** -7 * max(1.0, a[name].abs().max().item())
+        assert max_err(a[name], b[name]) <= tol, (name, max_err(a[name], b[name]))
 
 
 def test_c1_fp32_check_mode_against_cpu_eager(E):
