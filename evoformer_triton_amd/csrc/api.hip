@@ -59,7 +59,7 @@ static int bias_vec_ok(const EvoAttnParams &p) {
     return aligned(p.bias, a) && p.bias_stride_b % 4 == 0 && p.bias_stride_h % 4 == 0 && p.bias_stride_row % 4 == 0;
 }
 
-// The dQ kernel that double-buffers its operands in LDS keeps at most 4 key tiles per wave.
+// The dQ kernel that double-buffers its operands in LDS takes rows of limited length.
 static bool dq_ring_ok(const EvoAttnParams &p) {
     return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N <= mfma_dqr_max_n(p.D);
 }

@@ -292,34 +292,52 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 // ------------------------------------------------------------------ dK, dV (and dMask partials)
 //
 // Workgroup = NW (4 or 8) waves = NW*32 keys of one problem; each wave keeps its 32 keys' K and V
-// operands in registers and loops over all query rows, staged through LDS both row-major
-// (for S = Q K^T, dP = dO V^T) and transposed (for dV^T += dO^T P, dK^T += Q^T dS).
+// operands in registers and loops over all query rows.  Those are staged in LDS once,
+// row-major: Q pre-multiplied by scale*log2(e) exactly as in the forward, dO, and per query the
+// 16-bit columns that carry -LSE and -delta into the score MFMAs.  The transposed operands
+// of dV^T += dO^T P and dK^T += Q^T dS come from the same rows by transposing LDS reads
+// (`ds_read_b64_tr_b16`).  For head dims <= 16 the scaled Q is staged with its rounding residue
+// (as the scores need it), dK sums over both and is multiplied by scale / (scale*log2(e)) = ln 2
+// at the end; for the larger head dims Q is staged a second time as given and dK is
+// multiplied by scale (summing over the rounded scaled Q alone costs dK two digits at N = 768).
 // Scores are NOT transposed here: a lane owns one key and 16 queries, so that P and dS in
 // accumulator layout are the B operands of the two gradient matmuls.
-template <typename T, int D, bool HAS_BIAS, int NW>
+template <int D>
+struct KvGeo {
+    static constexpr int C = D / 8;                          // 16-byte chunks per row
+    static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
+    static constexpr int BQS = D <= 32 ? 256 : 128;          // query rows staged per round
+    static constexpr bool RESID = D <= 16;
+    // LDS layout for `rows` staged query rows (BQS, or 128 where a problem has no more):
+    //   [Q scaled][its rounding residue (RESID) or Q as given][dO][-LSE columns][-delta columns]
+    static __host__ __device__ constexpr int lds_bytes(int rows) { return rows * (3 * D * 2 + 32); }
+    static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
+};
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
 __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
-    constexpr int KW = G::KW, KS = G::KS, KSD = G::KSD, DT = G::DT, DP = G::DP, AUGC = G::AUGC;
+    typedef KvGeo<D> R;
+    constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
     constexpr int NTH = NW * 64;
     constexpr int BK = NW * 32;
     constexpr bool PREFETCH = NW == 4;       // the 8-wave form runs at 128 registers, 4 waves per SIMD
-    constexpr int BQS = D <= 32 ? 128 : 64;  // query rows staged per round
+    constexpr int BQS = ROWS, C = R::C;      // query rows staged per round
     constexpr int TPS = BQS / 32;            // query tiles per stage
-    constexpr int RW = G::RESID ? KSD * 16 : 0;  // residue columns of the scaled Q rows
-    constexpr int QP = KW + RW + 8;
-    constexpr int TP = BQS + 8;
     typedef typename Mfma<T>::v8 v8;
-    typedef typename Mfma<T>::v2 v2;
+    typedef typename Mfma<T>::v4 v4;
 
-    __shared__ __attribute__((aligned(16))) T Qs[BQS * QP];
-    __shared__ __attribute__((aligned(16))) T Gs[BQS * QP];
-    __shared__ __attribute__((aligned(16))) T Qt[DP * TP];
-    __shared__ __attribute__((aligned(16))) T Gt[DP * TP];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nkb = (p.N + BK - 1) / BK;
+    constexpr int srows = BQS;
+    constexpr int OFF_QS = 0, OFF_QL = srows * D * 2, OFF_QR = OFF_QL, OFF_G = 2 * OFF_QL;
+    constexpr int OFF_AQ = 3 * OFF_QL, OFF_AG = OFF_AQ + srows * 16;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nkb;
     const int key0 = (lid % nkb) * BK + wave * 32;
@@ -335,20 +353,6 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
     const float cs = p.scale * kLog2e;
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
-
-    // LDS that is read but never staged
-    if (!G::AUG_IN_PAD)
-        for (int r = tid; r < BQS; r += NTH) {
-            *reinterpret_cast<v8 *>(&Qs[r * QP + AUGC + 8]) = zero8<T>();
-            *reinterpret_cast<v8 *>(&Gs[r * QP + AUGC + 8]) = zero8<T>();
-        }
-    if (G::RESID && D < 16)
-        for (int r = tid; r < BQS; r += NTH) *reinterpret_cast<v8 *>(&Qs[r * QP + KW + 8]) = zero8<T>();
-    if (DP > D)
-        for (int i = tid; i < (DP - D) * TP / 8; i += NTH) {
-            *reinterpret_cast<v8 *>(&Qt[D * TP + i * 8]) = zero8<T>();
-            *reinterpret_cast<v8 *>(&Gt[D * TP + i * 8]) = zero8<T>();
-        }
 
     // this wave's keys: K with the mask columns, V with ones against -delta
     v8 kf[KS], vf[KS], kres[KSD];
@@ -395,41 +399,25 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
 
     auto stage = [&](int qs0) {
         __syncthreads();
-        for (int it = tid; it < BQS * (D / 8); it += NTH) {
-            const int row = it / (D / 8), ch = it % (D / 8), qq = qs0 + row;
+        for (int it = tid; it < srows * C; it += NTH) {
+            const int row = it / C, ch = it % C, qq = qs0 + row;
             v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + ch * 8) : zero8<T>();
             v8 bb2 = qq < p.N ? ld8(Gd + (int64_t)qq * sn + ch * 8) : zero8<T>();
             // the score operand carries scale*log2(e), rounded exactly as in the forward
             v8 hi, lo;
             scaled_hilo8<T>(a, cs, hi, lo);
-            *reinterpret_cast<v8 *>(&Qs[row * QP + ch * 8]) = hi;
-            if (G::RESID) *reinterpret_cast<v8 *>(&Qs[row * QP + KW + ch * 8]) = lo;
-            *reinterpret_cast<v8 *>(&Gs[row * QP + ch * 8]) = bb2;
+            const int o = R::swz(row, ch);
+            *reinterpret_cast<v8 *>(lds + OFF_QS + o) = hi;
+            *reinterpret_cast<v8 *>(lds + OFF_QL + o) = R::RESID ? lo : a;
+            *reinterpret_cast<v8 *>(lds + OFF_G + o) = bb2;
         }
-        for (int row = tid; row < BQS; row += NTH) {
+        for (int row = tid; row < srows; row += NTH) {
             const int qq = qs0 + row;
             // rows past N get -LSE = floor: their probabilities vanish
             const float nl = qq < p.N ? -p.lse[pr.row0 + qq] * kLog2e : kMaskFloor;
             const float nd = qq < p.N ? -e.delta[pr.row0 + qq] : 0.0f;
-            *reinterpret_cast<v8 *>(&Qs[row * QP + AUGC]) = aug8<T>(one3, pack_split3<T>(nl));
-            *reinterpret_cast<v8 *>(&Gs[row * QP + AUGC]) = aug8<T>(pack_split3<T>(nd), zero3);
-        }
-        constexpr int NPAIR = BQS / 2;
-        for (int it = tid; it < NPAIR * (D / 8); it += NTH) {
-            const int ch = it / NPAIR, jp = it % NPAIR, r0 = qs0 + 2 * jp;
-            v8 qa = r0 < p.N ? ld8(Q + (int64_t)r0 * sn + ch * 8) : zero8<T>();
-            v8 qb = r0 + 1 < p.N ? ld8(Q + (int64_t)(r0 + 1) * sn + ch * 8) : zero8<T>();
-            v8 ga = r0 < p.N ? ld8(Gd + (int64_t)r0 * sn + ch * 8) : zero8<T>();
-            v8 gb = r0 + 1 < p.N ? ld8(Gd + (int64_t)(r0 + 1) * sn + ch * 8) : zero8<T>();
-            const int pos = perm_pos(2 * jp);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                v2 w;
-                w[0] = qa[i]; w[1] = qb[i];
-                *reinterpret_cast<v2 *>(&Qt[(ch * 8 + i) * TP + pos]) = w;
-                w[0] = ga[i]; w[1] = gb[i];
-                *reinterpret_cast<v2 *>(&Gt[(ch * 8 + i) * TP + pos]) = w;
-            }
+            *reinterpret_cast<v8 *>(lds + OFF_AQ + row * 16) = aug8<T>(one3, pack_split3<T>(nl));
+            *reinterpret_cast<v8 *>(lds + OFF_AG + row * 16) = aug8<T>(pack_split3<T>(nd), zero3);
         }
         __syncthreads();
     };
@@ -442,8 +430,16 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
         for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            v8 qa = *reinterpret_cast<const v8 *>(&Qs[(qb + li) * QP + ks * 16 + g * 8]);
-            v8 ga = *reinterpret_cast<const v8 *>(&Gs[(qb + li) * QP + ks * 16 + g * 8]);
+            const int d0 = ks * 16 + g * 8;
+            v8 qa = zero8<T>(), ga = zero8<T>();
+            if (d0 < D) {
+                const int o = R::swz(qb + li, 2 * ks + g);
+                qa = *reinterpret_cast<const v8 *>(lds + OFF_QS + o);
+                ga = *reinterpret_cast<const v8 *>(lds + OFF_G + o);
+            } else if (d0 == AUGC) {
+                qa = *reinterpret_cast<const v8 *>(lds + OFF_AQ + (qb + li) * 16);
+                ga = *reinterpret_cast<const v8 *>(lds + OFF_AG + (qb + li) * 16);
+            }
             if (ks == 0) {
                 if (HAS_BIAS) {
                     acc = Mfma<T>::mma(qa, kf[0], ctile);
@@ -460,10 +456,11 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
         }
         // consumed above; with registers to spare the next tile travels during the rest
         if (PREFETCH) load_btile(qtile + 1, ctile);
-        if (G::RESID) {
+        if (R::RESID) {
 #pragma unroll
             for (int ks = 0; ks < KSD; ++ks) {
-                v8 ql = *reinterpret_cast<const v8 *>(&Qs[(qb + li) * QP + KW + ks * 16 + g * 8]);
+                v8 ql = zero8<T>();
+                if (ks * 16 + g * 8 < D) ql = *reinterpret_cast<const v8 *>(lds + OFF_QL + R::swz(qb + li, 2 * ks + g));
                 acc = Mfma<T>::mma(ql, kres[ks], acc);
             }
         }
@@ -491,10 +488,36 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                v8 ga = *reinterpret_cast<const v8 *>(&Gt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
-                v8 qa = *reinterpret_cast<const v8 *>(&Qt[(dt * 32 + li) * TP + qb + ts * 16 + g * 8]);
-                dv[dt] = Mfma<T>::mma(ga, pf, dv[dt]);
-                dk[dt] = Mfma<T>::mma(qa, dsf, dk[dt]);
+                // dO^T and Q^T fragments: row d = dt*32 + li, the 8 queries the P registers hold
+                const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                v8 gta = zero8<T>(), qta = zero8<T>(), qtl = zero8<T>();
+                if (col < D) {
+#pragma unroll
+                    for (int h2 = 0; h2 < 2; ++h2) {
+                        const int row = qb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                        const int o = R::swz(row, col >> 3) + (col & 7) * 2;
+                        s16x4 rg = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (s16x4 __attribute__((address_space(3))) *)(lds + OFF_G + o));
+                        s16x4 rq = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (s16x4 __attribute__((address_space(3))) *)(lds + (R::RESID ? OFF_QS : OFF_QR) + o));
+                        v4 vg = __builtin_bit_cast(v4, rg), vq = __builtin_bit_cast(v4, rq);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            gta[4 * h2 + i] = vg[i];
+                            qta[4 * h2 + i] = vq[i];
+                        }
+                        if (R::RESID) {
+                            s16x4 rl = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (s16x4 __attribute__((address_space(3))) *)(lds + OFF_QL + o));
+                            v4 vl = __builtin_bit_cast(v4, rl);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) qtl[4 * h2 + i] = vl[i];
+                        }
+                    }
+                }
+                dv[dt] = Mfma<T>::mma(gta, pf, dv[dt]);
+                dk[dt] = Mfma<T>::mma(qta, dsf, dk[dt]);
+                if (R::RESID) dk[dt] = Mfma<T>::mma(qtl, dsf, dk[dt]);
             }
         }
     };
@@ -515,14 +538,16 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
         if (key < p.N) {
             T *dK = (T *)p.dk + pr.base + (int64_t)key * sn;
             T *dV = (T *)p.dv + pr.base + (int64_t)key * sn;
+            // with the residue, dk holds the sum over Q * scale * log2(e)
+            const float kscale = R::RESID ? kLn2 : p.scale;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int d0 = dt * 32 + 8 * rr + 4 * g;
                     if (d0 < D) {
-                        store4<T>(dK + d0, dk[dt][4 * rr] * p.scale, dk[dt][4 * rr + 1] * p.scale,
-                                  dk[dt][4 * rr + 2] * p.scale, dk[dt][4 * rr + 3] * p.scale);
+                        store4<T>(dK + d0, dk[dt][4 * rr] * kscale, dk[dt][4 * rr + 1] * kscale,
+                                  dk[dt][4 * rr + 2] * kscale, dk[dt][4 * rr + 3] * kscale);
                         store4<T>(dV + d0, dv[dt][4 * rr], dv[dt][4 * rr + 1], dv[dt][4 * rr + 2], dv[dt][4 * rr + 3]);
                     }
                 }
@@ -553,16 +578,26 @@ static int dq_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 template <typename T, int D, int NW>
 static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned grid = (unsigned)((p.N + NW * 32 - 1) / (NW * 32)) * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW><<<grid, NW * 64, 0, st>>>(p, e);
-    else mfma_dkdv<T, D, true, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    typedef KvGeo<D> R;
+    if (NW == 4 && p.N <= 128) {
+        constexpr int lds = R::lds_bytes(128);
+        if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW, 128><<<grid, NW * 64, lds, st>>>(p, e);
+        else mfma_dkdv<T, D, true, NW, 128><<<grid, NW * 64, lds, st>>>(p, e);
+    } else {
+        constexpr int lds = R::lds_bytes(R::BQS);   // at most 56 KB
+        if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW, R::BQS><<<grid, NW * 64, lds, st>>>(p, e);
+        else mfma_dkdv<T, D, true, NW, R::BQS><<<grid, NW * 64, lds, st>>>(p, e);
+    }
     return hip_rc();
 }
 
-// 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys; worth it unless
-// the last workgroup of a problem would be more than half empty.
+// 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys: measured faster
+// (N = 256: 187 vs 211 us at S = 512, H = 8) unless the last workgroup of a problem would be
+// half empty or more (N = 384: 155 vs 141 us at S = 384, H = 4).
 template <typename T, int D>
 static int dkdv_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const bool wide = (p.flags & 0x100) != 0;   // measured slower than the 4-wave form at N = 256
+    // bit 0x100 of flags (not part of the public interface) inverts the choice, for comparison
+    const bool wide = (p.N > 128 && (p.N - 1) % 256 >= 128) != ((p.flags & 0x100) != 0);
     return wide ? dkdv_bias<T, D, 8>(p, e, st) : dkdv_bias<T, D, 4>(p, e, st);
 }
 

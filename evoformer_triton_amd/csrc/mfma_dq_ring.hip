@@ -150,14 +150,24 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     u32x4 stg[IPW];
     // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
-    auto piece = [&](int t, int n, const u32x4 *&src, int &dst) {
-        const int s = s_begin + t / NBLK, blk = t % NBLK;
+    // Where piece n of key block blk comes from and goes to: a base that every lane shares for
+    // the first S row of the chunk, its advance per S row (both in bytes), this lane's offset
+    // from it, and the LDS offset inside the stage.
+    struct Piece {
+        const unsigned char *base;
+        int64_t row_step;
+        unsigned lane_off;
+        int dst;
+    };
+    auto describe = [&](int n, int blk) {
+        Piece d;
         if (n >= 2 * R::I_K && n < R::I_KVA) {
             const int m = n - 2 * R::I_K;
-            src = reinterpret_cast<const u32x4 *>(e.m2a + ((int64_t)b * p.S + s) * np256 + blk * BKV + m * 64 + lane);
-            dst = R::OFF_A + m * 1024;
+            d.base = reinterpret_cast<const unsigned char *>(e.m2a + ((int64_t)b * p.S + s_begin) * np256 + blk * BKV + m * 64);
+            d.row_step = (int64_t)np256 * 16;
+            d.lane_off = lane * 16u;
+            d.dst = R::OFF_A + m * 1024;
         } else {
-            const int64_t pbase = base0 + (int64_t)(s - s_begin) * p.stride_s;
             const T *base;
             int m, row0, off;
             if (n < R::I_K) { base = (const T *)p.k; m = n; row0 = blk * BKV; off = 0; }
@@ -169,34 +179,41 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             const int r = L / C, cpos = L % C;
             const int ch = cpos ^ ((r / R::RPB) % C);
             const int row = min(row0 + r, p.N - 1);
-            src = reinterpret_cast<const u32x4 *>(base + pbase + (int64_t)(row * (int)sn + ch * 8));
-            dst = off + m * 1024;
+            d.base = reinterpret_cast<const unsigned char *>(base + base0);
+            d.row_step = p.stride_s * 2;
+            d.lane_off = (unsigned)(row * (int)sn + ch * 8) * 2u;
+            d.dst = off + m * 1024;
         }
+        return d;
     };
+    // With one key block per row the descriptors never change: form them once.  (With more
+    // they are re-formed per stage; that form only serves head dim 8.)
+    Piece fixed[NBLK == 1 ? IPW : 1];
+    if (NBLK == 1) {
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) fixed[i] = describe(min(wave + 8 * i, R::I_ALL - 1), 0);
+    }
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
     auto fetch = [&](int t) {
         t = min(t, T_total - 1);
-        const int ninst = (t % NBLK) == 0 ? R::I_ALL : R::I_KVA;
+        const int row = t / NBLK, blk = t % NBLK;
+        const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
-            const int n = min(wave + 8 * i, ninst - 1);
-            const u32x4 *src;
-            int dst;
-            piece(t, n, src, dst);
-            stg[i] = *src;
+            const Piece d = NBLK == 1 ? fixed[i] : describe(min(wave + 8 * i, ninst - 1), blk);
+            stg[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
         }
     };
     auto stash = [&](int t) {
-        const int ninst = t >= T_total ? 0 : (t % NBLK) == 0 ? R::I_ALL : R::I_KVA;
+        const int blk = t % NBLK;
+        const int ninst = t >= T_total ? 0 : blk == 0 ? R::I_ALL : R::I_KVA;
         unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             const int n = wave + 8 * i;
             if (n < ninst) {
-                const u32x4 *src;
-                int dst;
-                piece(min(t, T_total - 1), n, src, dst);
+                const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
                 *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
             }
         }
@@ -273,6 +290,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         gf[ks] = aug8<T>(pack_split3<T>(-dl), zero3);    // -delta x ones
                     }
                 }
+                if (kill) {  // no gradient through the scores of such a row: dP - delta := 0
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) gf[ks] = zero8<T>();
+                }
             }
 
             EVO_TR(4);
@@ -298,19 +319,25 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                                 va[ks] = aug8<T>(one3, zero3);                                                 // ones x -delta
                             }
                         }
-                        f32x16 acc, dp;
+                        f32x16 acc, dp, z;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) acc[r] = dp[r] = 0.0f;
-                        if (HAS_BIAS && !dead) acc = bres[slot];
+                        for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                        // the bias tile is the C operand of the first score MFMA (uniform branch)
+                        if (HAS_BIAS && !dead) acc = Mfma<T>::mma(ka[0], qf[0], bres[slot]);
+                        else acc = Mfma<T>::mma(ka[0], qf[0], z);
+                        dp = Mfma<T>::mma(va[0], gf[0], z);
+                        if (G::RESID) acc = Mfma<T>::mma(ka[0], qlo[0], acc);
 #pragma unroll
-                        for (int ks = 0; ks < KS; ++ks) {
+                        for (int ks = 1; ks < KS; ++ks) {
                             acc = Mfma<T>::mma(ka[ks], qf[ks], acc);   // log2 P^T
                             if (G::RESID && ks < KSD) acc = Mfma<T>::mma(ka[ks], qlo[ks], acc);
                             dp = Mfma<T>::mma(va[ks], gf[ks], dp);     // dP^T - delta
                         }
+                        // (in a row that a bool mask drops entirely dO and -delta were zeroed
+                        // above, so dP - delta and with it dS are zero)
                         float ds[16];
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) ds[r] = kill ? 0.0f : fast_exp2(acc[r]) * dp[r];
+                        for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(acc[r]) * dp[r];
 #pragma unroll
                         for (int ts = 0; ts < 2; ++ts) {
                             v8 dsf;
@@ -424,16 +451,19 @@ static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return hip_rc();
 }
 
+// Key blocks per row the kernel is built for: with more, the resident bias tiles and dBias
+// accumulators (16 registers each per key tile and wave) no longer fit 256 registers, and the
+// spilled form measured slower than the one-workgroup-per-problem kernel (N = 384, D = 32).
+template <int D>
+constexpr int dqr_max_blocks() { return D == 8 ? 2 : 1; }
+
 template <typename T, int D, bool HAS_BIAS>
 static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     typedef RingGeo<D> R;
     const int nblk = (p.N + R::BKV - 1) / R::BKV;
-    if (nblk * R::TPW > 4) return EVO_EUNSUPPORTED;
     if (nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1>(p, e, st);
-    if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2>(p, e, st);
-    if constexpr (R::TPW == 1) {
-        if (nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3>(p, e, st);
-        if (nblk == 4) return dqr_launch<T, D, HAS_BIAS, 4>(p, e, st);
+    if constexpr (dqr_max_blocks<D>() >= 2) {
+        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2>(p, e, st);
     }
     return EVO_EUNSUPPORTED;
 }
@@ -443,8 +473,8 @@ static int dqr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.bias_dtype == EVO_NONE ? dqr_blocks<T, D, false>(p, e, st) : dqr_blocks<T, D, true>(p, e, st);
 }
 
-// Largest N the double-buffered dQ kernel takes for this head dim (4 key tiles per wave).
-int EVO_CAT(mfma_dqr_max_n_d, EVO_D)() { return 4 / RingGeo<EVO_D>::TPW * RingGeo<EVO_D>::BKV; }
+// Largest N the double-buffered dQ kernel takes for this head dim.
+int EVO_CAT(mfma_dqr_max_n_d, EVO_D)() { return dqr_max_blocks<EVO_D>() * RingGeo<EVO_D>::BKV; }
 
 int EVO_CAT(launch_mfma_dqr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.dtype == EVO_BF16 ? dqr_bias<bf16_t, EVO_D>(p, e, st) : dqr_bias<f16_t, EVO_D>(p, e, st);
