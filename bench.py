@@ -31,6 +31,13 @@ if ROOT not in sys.path:
 
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch (reads + writes) from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE),
+# each scaled by what the counter reads for a plain 256 MiB copy (2.000 and 1.000); the runs
+# and their raw readings are in profiles/mfma_kernels_C2_hbm_traffic.md.  Not measurable from
+# inside this script, so only the profiled workload has a figure.
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    ("C2", "mfma_fwd_ring"): 367.1e6, ("C2", "mfma_dq_ring"): 480.4e6, ("C2", "mfma_dkdv"): 486.9e6,
+}
 
 
 def parse():
@@ -191,7 +198,8 @@ def main():
         "kernel_ms": {kernel_names[n]: t * 1e3 for n, t in t_phase.items()},
         "peak_mem_bytes_beyond_inputs": int(peak_extra),
         "roofline": {"bound": "mfma", "kernel": kernel_names[dom], "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
+                     "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, kernel_names[dom].split("+")[-1])),
                      "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3},
     }
     if not args.no_cpu_baseline:
