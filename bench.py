@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2]
 
 One "step" is one forward + backward of the attention over one batch of synthetic input
-(BASELINE configuration C2 by default: MSA row attention, Q,K,V [1,512,256,8,32] bf16,
+(benchmark configuration C2 by default: MSA row attention, Q,K,V [1,512,256,8,32] bf16,
 additive row mask, bf16 pair bias), called through the public operator
 `EvoformerAttention.apply` + autograd, inputs resident in HBM.  Prints ONE JSON line.
 
@@ -32,8 +32,8 @@ if ROOT not in sys.path:
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (reads + writes) from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the counter reads for a plain 256 MiB copy (2.000 and 1.000); the runs
-# and their raw readings are in profiles/mfma_kernels_C2_hbm_traffic.md.  Not measurable from
+# each scaled by what the counter reads for a plain 256 MiB copy (2.000 and 1.000); the commands
+# and raw readings are kept with the other profile summaries.  Not measurable from
 # inside this script, so only the profiled workload has a figure.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     ("C2", "mfma_fwd_ring"): 367.1e6, ("C2", "mfma_dq_ring"): 480.4e6, ("C2", "mfma_dkdv"): 486.9e6,
@@ -81,7 +81,7 @@ def main():
     args = parse()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
-              "(the path shards over S with one dBias all-reduce, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard over S with one dBias all-reduce)", file=sys.stderr)
         sys.exit(2)
     import torch
     from oracle import eager

@@ -1,6 +1,6 @@
 """GPU parity: the HIP path, called through the C ABI, against the oracle.
 
-Tolerances (BASELINE north_star): max-abs <= 2e-2 for bf16, <= 1e-5 for the fp32 check
+Tolerances: max-abs <= 2e-2 for bf16, <= 1e-5 for the fp32 check
 mode, on O, dQ, dK, dV, dBias; plus the reference's own criterion
 allclose(atol=1e-2, rtol=1e-2) (dsevoformer-triton/test.py:73-80) on its own shape matrix.
 Small cases use the oracle on the CPU and the committed golden fixtures; full-size cases
@@ -464,7 +464,7 @@ def test_full_size_properties_c2(E):
 
 def test_score_memory_is_linear_in_n(E):
     """Peak device memory of one fwd+bwd beyond inputs and outputs: LSE, delta, the dBias
-    partials and small vectors only; nothing of size [S,N,N] (BASELINE C3 vs C4)."""
+    partials and small vectors only; nothing of size [S,N,N] (configurations C3 vs C4)."""
     from evoformer_triton_amd import _lib
     lib = _lib.load()
     extra = {}
