@@ -203,7 +203,7 @@ const char *evoattn_path(const EvoAttnParams *p, int pass) {
     return mfma_ok(*p, pass) ? "mfma" : "generic";
 }
 
-// rows of 129..256 keys: a workgroup per chunk of S rows with the bias tiles resident
+// rows of 129..256 keys: a workgroup per chunk of S rows with the head's bias resident
 static bool fwd_ring_ok(const EvoAttnParams &p) {
     return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
 }

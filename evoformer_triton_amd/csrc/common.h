@@ -240,4 +240,27 @@ __device__ __forceinline__ void store4(T *dst, float a, float b, float c, float 
     *reinterpret_cast<typename Mfma<T>::v4 *>(dst) = v;
 }
 
+// One accumulator tile's worth of a row to memory as T: lane (li, g) holds, for its row, the
+// 16 values of columns 8 (r / 4) + 4 g + r % 4; the two lanes of a row exchange halves so
+// that each stores 16 contiguous bytes (columns c0 + 16 p + 8 g .. + 7, p = 0, 1) instead of
+// four 8-byte pieces.  Columns at or beyond `ncols` are not stored.
+template <typename T>
+__device__ __forceinline__ void store_row_tile(T *row, int c0, int ncols, const f32x16 &acc, float scale, int g) {
+#pragma unroll
+    for (int pp = 0; pp < 2; ++pp) {
+        typename Mfma<T>::v4 x, y;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[i] = (T)(acc[8 * pp + i] * scale);
+            y[i] = (T)(acc[8 * pp + 4 + i] * scale);
+        }
+        const uint2 xu = __builtin_bit_cast(uint2, x), yu = __builtin_bit_cast(uint2, y);
+        // lanes 32..63 of the first operand trade places with lanes 0..31 of the second
+        auto s0 = __builtin_amdgcn_permlane32_swap(xu.x, yu.x, false, false);
+        auto s1 = __builtin_amdgcn_permlane32_swap(xu.y, yu.y, false, false);
+        const int c = c0 + 16 * pp + 8 * g;
+        if (c < ncols) *reinterpret_cast<uint4 *>(row + c) = make_uint4(s0[0], s1[0], s0[1], s1[1]);
+    }
+}
+
 }  // namespace evo

@@ -316,6 +316,16 @@ struct KvGeo {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
+#ifdef EVO_TRACE
+#define EVO_TK(slot)                                                                             \
+    do {                                                                                         \
+        if (e.trace && (threadIdx.x & 63) == 0)                                                  \
+            e.trace[((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define EVO_TK(slot) do {} while (0)
+#endif
+
 template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
 __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
@@ -323,7 +333,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
     constexpr int NTH = NW * 64;
     constexpr int BK = NW * 32;
-    constexpr bool PREFETCH = NW == 4;       // the 8-wave form runs at 128 registers, 4 waves per SIMD
+    constexpr bool PREFETCH = NW == 4;       // the 8-wave form runs at 128 registers: prefetching there spills (227 vs 187 us)
     constexpr int BQS = ROWS, C = R::C;      // query rows staged per round
     constexpr int TPS = BQS / 32;            // query tiles per stage
     typedef typename Mfma<T>::v8 v8;
@@ -331,6 +341,7 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
+    EVO_TK(0);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
@@ -354,25 +365,17 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
 
-    // this wave's keys: K with the mask columns, V with ones against -delta
-    v8 kf[KS], vf[KS], kres[KSD];
+    // this wave's keys: requested now, used after the queries have been staged, so that the
+    // two round trips to memory overlap
+    v8 kraw[KSD], vraw[KSD];
 #pragma unroll
-    for (int ks = 0; ks < KSD; ++ks) kres[ks] = zero8<T>();
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-        const int d0 = ks * 16 + g * 8;
-        kf[ks] = zero8<T>();
-        vf[ks] = zero8<T>();
-        if (d0 < D) {
-            if (!dead) kf[ks] = ld8(K + (int64_t)keyc * sn + d0);
-            if (ks < KSD) kres[ks] = kf[ks];   // against the residue columns of Q: data only
-            vf[ks] = ld8(V + (int64_t)keyc * sn + d0);
-        } else if (d0 == AUGC) {
-            const int kk = min(key, npad - 1);
-            kf[ks] = aug8<T>(e.m2[((int64_t)pr.b * p.S + pr.s) * npad + kk], one3);  // mask x ones, ones x -lse
-            vf[ks] = aug8<T>(one3, zero3);                                           // ones x -delta
-        }
+    for (int ks = 0; ks < KSD; ++ks) {
+        const int d0 = min(ks * 16 + g * 8, D - 8);
+        kraw[ks] = ld8(K + (int64_t)keyc * sn + d0);
+        vraw[ks] = ld8(V + (int64_t)keyc * sn + d0);
     }
+    const uint2 mraw = e.m2[((int64_t)pr.b * p.S + pr.s) * npad + min(key, npad - 1)];
+    v8 kf[KS], vf[KS], kres[KSD];   // the operands built from them
 
     const int bb = e.bias_batches > 1 ? pr.b : 0;
     const int ktc = min(key0 >> 5, NT - 1);
@@ -398,18 +401,35 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
     float dm = 0.0f;
 
     auto stage = [&](int qs0) {
+        EVO_TK(1);
         __syncthreads();
-        for (int it = tid; it < srows * C; it += NTH) {
-            const int row = it / C, ch = it % C, qq = qs0 + row;
-            v8 a = qq < p.N ? ld8(Q + (int64_t)qq * sn + ch * 8) : zero8<T>();
-            v8 bb2 = qq < p.N ? ld8(Gd + (int64_t)qq * sn + ch * 8) : zero8<T>();
-            // the score operand carries scale*log2(e), rounded exactly as in the forward
-            v8 hi, lo;
-            scaled_hilo8<T>(a, cs, hi, lo);
-            const int o = R::swz(row, ch);
-            *reinterpret_cast<v8 *>(lds + OFF_QS + o) = hi;
-            *reinterpret_cast<v8 *>(lds + OFF_QL + o) = R::RESID ? lo : a;
-            *reinterpret_cast<v8 *>(lds + OFF_G + o) = bb2;
+        EVO_TK(2);
+        // all loads first, then the conversions and LDS writes: one round trip, not one per piece
+        constexpr int NIT = (srows * C + NTH - 1) / NTH;
+        v8 qv[NIT], gv[NIT];
+#pragma unroll
+        for (int i = 0; i < NIT; ++i) {
+            const int it = tid + i * NTH;
+            const int row = min(it / C, srows - 1), ch = it % C, qq = min(qs0 + row, p.N - 1);
+            qv[i] = ld8(Q + (int64_t)qq * sn + ch * 8);
+            gv[i] = ld8(Gd + (int64_t)qq * sn + ch * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NIT; ++i) {
+            const int it = tid + i * NTH;
+            if (it < srows * C) {
+                const int row = it / C, ch = it % C;
+                const bool in = qs0 + row < p.N;
+                const v8 a = in ? qv[i] : zero8<T>();
+                const v8 bb2 = in ? gv[i] : zero8<T>();
+                // the score operand carries scale*log2(e), rounded exactly as in the forward
+                v8 hi, lo;
+                scaled_hilo8<T>(a, cs, hi, lo);
+                const int o = R::swz(row, ch);
+                *reinterpret_cast<v8 *>(lds + OFF_QS + o) = hi;
+                *reinterpret_cast<v8 *>(lds + OFF_QL + o) = R::RESID ? lo : a;
+                *reinterpret_cast<v8 *>(lds + OFF_G + o) = bb2;
+            }
         }
         for (int row = tid; row < srows; row += NTH) {
             const int qq = qs0 + row;
@@ -419,7 +439,9 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
             *reinterpret_cast<v8 *>(lds + OFF_AQ + row * 16) = aug8<T>(one3, pack_split3<T>(nl));
             *reinterpret_cast<v8 *>(lds + OFF_AG + row * 16) = aug8<T>(pack_split3<T>(nd), zero3);
         }
+        EVO_TK(3);
         __syncthreads();
+        EVO_TK(4);
     };
 
     // one 32-query tile against this wave's 32 keys
@@ -524,10 +546,29 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
 
     f32x16 ctile;
     if (PREFETCH) load_btile(0, ctile);
+    stage(0);
+    // K with the mask columns, V with ones against -delta
+#pragma unroll
+    for (int ks = 0; ks < KSD; ++ks) kres[ks] = zero8<T>();
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = ks * 16 + g * 8;
+        kf[ks] = zero8<T>();
+        vf[ks] = zero8<T>();
+        if (d0 < D) {
+            if (!dead) kf[ks] = kraw[ks];
+            if (ks < KSD) kres[ks] = kf[ks];   // against the residue columns of Q: data only
+            vf[ks] = vraw[ks];
+        } else if (d0 == AUGC) {
+            kf[ks] = aug8<T>(mraw, one3);      // mask x ones, ones x -lse
+            vf[ks] = aug8<T>(one3, zero3);     // ones x -delta
+        }
+    }
     for (int qtile = 0; qtile < NT; ++qtile) {
-        if (qtile % TPS == 0) stage(qtile * 32);
+        if (qtile % TPS == 0 && qtile != 0) stage(qtile * 32);
         if (!PREFETCH) load_btile(qtile, ctile);
         if (active) compute(qtile, ctile);
+        if (qtile < 8) EVO_TK(5 + qtile);
     }
 
     if (active) {
@@ -541,18 +582,13 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
             // with the residue, dk holds the sum over Q * scale * log2(e)
             const float kscale = R::RESID ? kLn2 : p.scale;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int d0 = dt * 32 + 8 * rr + 4 * g;
-                    if (d0 < D) {
-                        store4<T>(dK + d0, dk[dt][4 * rr] * kscale, dk[dt][4 * rr + 1] * kscale,
-                                  dk[dt][4 * rr + 2] * kscale, dk[dt][4 * rr + 3] * kscale);
-                        store4<T>(dV + d0, dv[dt][4 * rr], dv[dt][4 * rr + 1], dv[dt][4 * rr + 2], dv[dt][4 * rr + 3]);
-                    }
-                }
+            for (int dt = 0; dt < DT; ++dt) {
+                store_row_tile<T>(dK, dt * 32, D, dk[dt], kscale, g);
+                store_row_tile<T>(dV, dt * 32, D, dv[dt], 1.0f, g);
+            }
         }
     }
+    EVO_TK(13);
 }
 
 // ------------------------------------------------------------------ launchers
@@ -592,12 +628,12 @@ static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 }
 
 // 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys: measured faster
-// (N = 256: 187 vs 211 us at S = 512, H = 8) unless the last workgroup of a problem would be
-// half empty or more (N = 384: 155 vs 141 us at S = 384, H = 4).
+// wherever a problem has more than 128 keys (N = 256: 171 vs 191 us at S = 512, H = 8;
+// N = 384, D = 32: 127 vs 149 us; N = 384, D = 8 within 3 %).
 template <typename T, int D>
 static int dkdv_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     // bit 0x100 of flags (not part of the public interface) inverts the choice, for comparison
-    const bool wide = (p.N > 128 && (p.N - 1) % 256 >= 128) != ((p.flags & 0x100) != 0);
+    const bool wide = (p.N > 128) != ((p.flags & 0x100) != 0);
     return wide ? dkdv_bias<T, D, 8>(p, e, st) : dkdv_bias<T, D, 4>(p, e, st);
 }
 

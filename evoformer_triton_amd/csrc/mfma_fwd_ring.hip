@@ -1,21 +1,30 @@
 // Forward for rows of at most 256 keys: one workgroup walks over a chunk of S rows of one
-// head with the head's bias tiles resident in registers.  Compiled once per head dim.
+// head with the head's bias resident in registers.  Compiled once per head dim.
 //
 // Same arithmetic as mfma_fwd.hip (the reference's `_attn_fwd`, evoformer.py:23-297).  That
 // kernel is one workgroup per (b, h, s) problem: every problem starts with loads whose
 // latency nothing hides, and every problem reads its N x N bias tiles again (fp32, from L2),
 // which at N = 256, D = 32 is four times the bytes of Q, K, V and O together.  Here
 //   * a workgroup has 8 waves = 256 query rows (all of them) and a fixed head; wave w keeps
-//     the bias tiles (query tile w) x (key tiles 0..7) in 128 registers for the whole chunk
-//     of S rows, so the bias is read once per chunk instead of once per row;
+//     the bias of (query tile w) x (all keys) for the whole chunk of S rows, as it sits in
+//     memory: 16-bit values, 64 registers, read once per chunk straight from the caller's
+//     tensor.  It enters the scores through the matrix core, S^T += (I c) B^T with I the
+//     identity and c = log2(e) as hi + lo of the 16-bit type (4 MFMAs per 32 x 32 tile on a
+//     unit that is mostly idle; exact to 2^-17);
 //   * K, V and the mask columns of row s+1 are requested (16 bytes per lane and load) before
 //     row s is computed out of one LDS buffer and written into the other one afterwards; a
 //     wave's own Q rows are prefetched straight into its registers;
+//   * the running maximum is folded into the next step's score MFMA as three more 16-bit
+//     columns (next to the mask's), so that the scores arrive relative to it and the common
+//     step does no subtraction; row sums are taken from the converted pairs (`v_dot2c`),
+//     i.e. of exactly the probabilities that multiply V;
 //   * V^T fragments come from row-major V by transposing LDS reads (`ds_read_b64_tr_b16`);
 //   * one workgroup barrier per S row.
 // K and V rows sit in LDS row-major without padding; 16-byte chunks are XOR-swizzled by row
 // so that the operand reads and the transposing reads are free of bank conflicts.
-#include "common.h"
+// Needs the bias in the inputs' dtype with 16-byte aligned rows (N % 8 == 0); other cases
+// run mfma_fwd.hip.
+#include "bwd_common.h"
 #include "kernels.h"
 
 #ifndef EVO_D
@@ -48,7 +57,48 @@ struct FwdRingGeo {
 // of the last one stay in flight across it (__syncthreads() would wait for them).
 __device__ __forceinline__ void lds_barrier_f() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <typename T, int D, bool HAS_BIAS>
+#ifdef EVO_TRACE
+#define EVO_TR(slot)                                                                             \
+    do {                                                                                         \
+        if (e.trace && (threadIdx.x & 63) == 0 && t == 3)                                        \
+            e.trace[((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define EVO_TR(slot) do {} while (0)
+#endif
+
+// acc + the sum of the eight 16-bit values of x, two per instruction.
+template <typename T>
+__device__ __forceinline__ float pair_sums(typename Mfma<T>::v8 x, float acc);
+template <>
+__device__ __forceinline__ float pair_sums<bf16_t>(bf16x8 x, float acc) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 one;
+    one[0] = one[1] = (__bf16)1.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bf2 v;
+        v[0] = x[2 * i]; v[1] = x[2 * i + 1];
+        acc = __builtin_amdgcn_fdot2_f32_bf16(v, one, acc, false);
+    }
+    return acc;
+}
+template <>
+__device__ __forceinline__ float pair_sums<f16_t>(f16x8 x, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 one;
+    one[0] = one[1] = (_Float16)1.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        h2 v;
+        v[0] = x[2 * i]; v[1] = x[2 * i + 1];
+        acc = __builtin_amdgcn_fdot2(v, one, acc, false);
+    }
+    return acc;
+}
+
+// BIASK: 0 no bias, 1 fp32 tiles (x log2(e), accumulator order) as C operands, 2 the caller's 16-bit rows through the identity
+template <typename T, int D, int BIASK>
 __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     typedef FwdRingGeo<D> R;
     constexpr int C = R::C;
@@ -79,8 +129,11 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     const int64_t sn = p.stride_n;
     const float cscale = p.scale * kLog2e;
 
-    f32x16 bres[HAS_BIAS ? 8 : 1];
-    if (HAS_BIAS) {
+    // bias of this wave's query rows, as B operands: lane = query li, k-step (j, ks) holds keys
+    // 32 j + 16 ks + 8 g .. + 7
+    v8 bres[BIASK == 2 ? 16 : 1];
+    f32x16 btile[BIASK == 1 ? 8 : 1];
+    if (BIASK == 1) {
         const int bb = e.bias_batches > 1 ? b : 0;
         const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + min(wave, NT - 1)) * NT) * 1024 + lane * 16;
 #pragma unroll
@@ -89,8 +142,33 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
-                bres[j][4 * rr] = v[0]; bres[j][4 * rr + 1] = v[1]; bres[j][4 * rr + 2] = v[2]; bres[j][4 * rr + 3] = v[3];
+                btile[j][4 * rr] = v[0]; btile[j][4 * rr + 1] = v[1]; btile[j][4 * rr + 2] = v[2]; btile[j][4 * rr + 3] = v[3];
             }
+        }
+    }
+    // (identity x log2(e)) as A operands, hi and lo parts: row = key li of the tile, column 16 ks + 8 g + i
+    v8 idh[2], idl[2];
+    {
+        const T chi = (T)kLog2e;
+        const T clo = (T)(kLog2e - (float)chi);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool on = li == 16 * ks + 8 * g + i;
+                idh[ks][i] = on ? chi : (T)0.0f;
+                idl[ks][i] = on ? clo : (T)0.0f;
+            }
+    }
+    if (BIASK == 2) {
+        const int bb = e.bias_batches > 1 ? b : 0;
+        const T *brow = (const T *)p.bias + (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h +
+                        (int64_t)qrow * p.bias_stride_row;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            // chunks past the row repeat its last one (those keys carry the mask floor)
+            const int key0 = min((j >> 1) * 32 + 16 * (j & 1) + 8 * g, p.N - 8);
+            bres[j] = ld8(brow + key0);
         }
     }
 
@@ -101,14 +179,30 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
 
     // ---- the stage of row s_begin + t lives in buffer t & 1.  It is a list of 1 KB pieces
-    // (64 lanes x 16 bytes); piece n belongs to wave n % 8.  Lane i of piece m of K or V fills
-    // LDS slot 64 m + i of that block, which the swizzle assigns to some chunk of some row.
+    // (64 lanes x 16 bytes): K, V, then the mask columns; piece n belongs to wave n % 8.  Lane
+    // i of piece m of K or V fills LDS slot 64 m + i of that block, which the swizzle assigns
+    // to some chunk of some row.
     u32x4 stg[IPW];
-    auto piece = [&](int t, int n, const u32x4 *&src, int &dst) {
+    // Where a piece comes from and goes to: a base that every lane shares for the first row
+    // of the chunk, its advance per S row (both in bytes), this lane's offset from it, and
+    // the LDS offset inside the stage.  They never change, so they are formed once.
+    struct Piece {
+        const unsigned char *base;
+        int64_t row_step;
+        unsigned lane_off;
+        int dst;
+    };
+    Piece pc[IPW];
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) {
+        // (a wave with fewer pieces repeats its last one)
+        const int n = min(wave + 8 * i, R::I_ALL - 1);
         if (n >= 2 * R::I_K) {
             const int m = n - 2 * R::I_K;
-            src = reinterpret_cast<const u32x4 *>(e.m2a + ((int64_t)b * p.S + s_begin + t) * np256 + m * 64 + lane);
-            dst = R::OFF_A + m * 1024;
+            pc[i].base = reinterpret_cast<const unsigned char *>(e.m2a + ((int64_t)b * p.S + s_begin) * np256 + m * 64);
+            pc[i].row_step = (int64_t)np256 * 16;
+            pc[i].lane_off = lane * 16u;
+            pc[i].dst = R::OFF_A + m * 1024;
         } else {
             const bool isv = n >= R::I_K;
             const int m = isv ? n - R::I_K : n;
@@ -117,36 +211,26 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
             const int r = L / C, cpos = L % C;
             const int ch = cpos ^ ((r / R::RPB) % C);
             const int row = min(r, p.N - 1);
-            src = reinterpret_cast<const u32x4 *>(base + base0 + (int64_t)t * p.stride_s + (int64_t)(row * (int)sn + ch * 8));
-            dst = (isv ? R::OFF_V : 0) + m * 1024;
+            pc[i].base = reinterpret_cast<const unsigned char *>(base + base0);
+            pc[i].row_step = p.stride_s * 2;
+            pc[i].lane_off = (unsigned)(row * (int)sn + ch * 8) * 2u;
+            pc[i].dst = (isv ? R::OFF_V : 0) + m * 1024;
         }
-    };
-    // Loads are unconditional (a wave with fewer pieces repeats its last one, the row past the
-    // end repeats the last row) so that the staging registers stay registers.
+    }
+    // Loads are unconditional (the row past the end repeats the last row) so that the
+    // staging registers stay registers.
     auto fetch = [&](int t) {
         t = min(t, nrows - 1);
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) {
-            const int n = min(wave + 8 * i, R::I_ALL - 1);
-            const u32x4 *src;
-            int dst;
-            piece(t, n, src, dst);
-            stg[i] = *src;
-        }
+        for (int i = 0; i < IPW; ++i)
+            stg[i] = *reinterpret_cast<const u32x4 *>(pc[i].base + t * pc[i].row_step + pc[i].lane_off);
     };
     auto stash = [&](int t) {
         if (t >= nrows) return;
         unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) {
-            const int n = wave + 8 * i;
-            if (n < R::I_ALL) {
-                const u32x4 *src;
-                int dst;
-                piece(t, n, src, dst);
-                *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
-            }
-        }
+        for (int i = 0; i < IPW; ++i)
+            if (wave + 8 * i < R::I_ALL) *reinterpret_cast<u32x4 *>(buf + pc[i].dst + lane * 16) = stg[i];
     };
     // this lane's half of its query row, straight from global memory
     v8 qraw[KSD], qnext[KSD];
@@ -168,9 +252,12 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         const int s = s_begin + t;
         const unsigned pid = bh * (unsigned)p.S + s;
         const bool dead = e.dead[b * p.S + s] != 0;
+        EVO_TR(0);
         lds_barrier_f();   // the stage of this row is in LDS; everybody is done with the row before
+        EVO_TR(1);
         fetch(t + 1);
         fetch_q(t + 1, qnext);
+        EVO_TR(2);
         const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 
         if (qact) {
@@ -182,121 +269,165 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 qlo[ks] = zero8<T>();
                 if (2 * ks + g < C) scaled_hilo8<T>(qraw[ks], cq, qf[ks], qlo[ks]);
             }
-            float m = -INFINITY, l = 0.0f;
+            // m: the maximum the probabilities are relative to; mf: what the mask k-step
+            // currently subtracts inside the MFMA (m, or 0 while m is not yet known or too
+            // large to be carried in three 16-bit columns next to scores of order one)
+            float m = 0.0f, mf = 0.0f, l = 0.0f;
+            v8 qaug = aug8<T>(ones3<T>(), uint2{0u, 0u});   // ones x mask columns, -mf x ones
             f32x16 oacc[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.0f;
 
+            // ---- scores of one 64-key step: S^T = bias^T log2(e) + K Q^T + mask - mf
+            auto scores = [&](int step, f32x16 &a0, f32x16 &a1) {
+                const int kb = step * 64;
+                bool started = false;
+                if (BIASK == 2 && !dead) {  // uniform
+                    f32x16 z;
 #pragma unroll
-            for (int step = 0; step < 4; ++step) {
-                if (step < nsteps) {  // uniform
-                    const int kb = step * 64;
-                    // ---- scores: S^T = K Q^T (+ bias tiles as C, + mask columns)
-                    f32x16 a0, a1;
+                    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                    a0 = Mfma<T>::mma(idh[0], bres[4 * step], z);
+                    a1 = Mfma<T>::mma(idh[0], bres[4 * step + 2], z);
+                    a0 = Mfma<T>::mma(idl[0], bres[4 * step], a0);
+                    a1 = Mfma<T>::mma(idl[0], bres[4 * step + 2], a1);
+                    a0 = Mfma<T>::mma(idh[1], bres[4 * step + 1], a0);
+                    a1 = Mfma<T>::mma(idh[1], bres[4 * step + 3], a1);
+                    a0 = Mfma<T>::mma(idl[1], bres[4 * step + 1], a0);
+                    a1 = Mfma<T>::mma(idl[1], bres[4 * step + 3], a1);
+                    started = true;
+                }
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-                        v8 k0, k1, qb;
-                        if (ks < KSD) {
-                            const int ch = 2 * ks + g;
-                            if (AUG_IN_PAD && g == 1) {
-                                k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
-                                k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
-                                qb = zero8<T>();
-                                qb[0] = qb[1] = qb[2] = (T)1.0f;
-                            } else {
-                                k0 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + li, ch < C ? ch : 0));
-                                k1 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + 32 + li, ch < C ? ch : 0));
-                                qb = qf[ks];
-                            }
-                        } else {  // the mask k-step: columns 0..2 of lane group 0
-                            k0 = zero8<T>();
-                            k1 = zero8<T>();
-                            qb = zero8<T>();
-                            if (g == 0) {
-                                k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
-                                k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
-                                qb[0] = qb[1] = qb[2] = (T)1.0f;
-                            }
-                        }
-                        if (ks == 0) {
-                            f32x16 z;
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) z[r] = 0.0f;
-                            if (HAS_BIAS && !dead) {  // uniform
-                                a0 = Mfma<T>::mma(k0, qb, bres[2 * step]);
-                                a1 = Mfma<T>::mma(k1, qb, bres[2 * step + 1]);
-                            } else {
-                                a0 = Mfma<T>::mma(k0, qb, z);
-                                a1 = Mfma<T>::mma(k1, qb, z);
-                            }
+                for (int ks = 0; ks < KS; ++ks) {
+                    v8 k0, k1, qb;
+                    if (ks < KSD) {
+                        const int ch = 2 * ks + g;
+                        if (AUG_IN_PAD && g == 1) {
+                            k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
+                            k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
+                            qb = qaug;
                         } else {
-                            a0 = Mfma<T>::mma(k0, qb, a0);
-                            a1 = Mfma<T>::mma(k1, qb, a1);
+                            k0 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + li, ch < C ? ch : 0));
+                            k1 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + 32 + li, ch < C ? ch : 0));
+                            qb = qf[ks];
                         }
-                        if (RESID && ks < KSD) {
-                            v8 ql = (AUG_IN_PAD && g == 1) ? zero8<T>() : qlo[ks];
-                            a0 = Mfma<T>::mma(k0, ql, a0);
-                            a1 = Mfma<T>::mma(k1, ql, a1);
+                    } else {  // the mask k-step: lane group 0
+                        k0 = zero8<T>();
+                        k1 = zero8<T>();
+                        qb = zero8<T>();
+                        if (g == 0) {
+                            k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
+                            k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
+                            qb = qaug;
                         }
                     }
-                    // ---- online softmax
-                    float mloc = fmaxf(a0[0], a1[0]);
+                    if (ks == 0 && BIASK == 1 && !dead) {  // uniform
+                        a0 = Mfma<T>::mma(k0, qb, btile[2 * step]);
+                        a1 = Mfma<T>::mma(k1, qb, btile[2 * step + 1]);
+                    } else if (ks == 0 && !started) {
+                        f32x16 z;
 #pragma unroll
-                    for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
-                    {   // exchange between the two lane groups without touching LDS
-                        const unsigned u = __float_as_uint(mloc);
-                        auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-                        mloc = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                        for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                        a0 = Mfma<T>::mma(k0, qb, z);
+                        a1 = Mfma<T>::mma(k1, qb, z);
+                    } else {
+                        a0 = Mfma<T>::mma(k0, qb, a0);
+                        a1 = Mfma<T>::mma(k1, qb, a1);
                     }
-                    // rescale only when the max grows by more than 2^TAU
-                    const bool grow = mloc > m + TAU;
-                    if (__any(grow)) {
-                        const float mn = grow ? mloc : m;
-                        const float alpha = fast_exp2(m - mn);
+                    if (RESID && ks < KSD) {
+                        v8 ql = (AUG_IN_PAD && g == 1) ? zero8<T>() : qlo[ks];
+                        a0 = Mfma<T>::mma(k0, ql, a0);
+                        a1 = Mfma<T>::mma(k1, ql, a1);
+                    }
+                }
+            };
+            // ---- online softmax of one step, part 1: where the maximum stands.  `used` is the
+            // mf the step's scores were formed with (they are relative to it).
+            auto settle = [&](int step, f32x16 &a0, f32x16 &a1, float used) {
+                float mloc = fmaxf(a0[0], a1[0]);
+#pragma unroll
+                for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
+                {   // exchange between the two lane groups without touching LDS
+                    const unsigned u = __float_as_uint(mloc);
+                    auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+                    mloc = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+                }
+                const float cand = mloc + used;
+                // move m only when the maximum grows by more than 2^TAU (always at the first step)
+                const bool grow = step == 0 || cand > m + TAU;
+                if (__any(grow || m != used)) {
+                    const float mn = grow ? cand : m;
+                    if (step != 0) {
+                        const float alpha = fast_exp2(m - mn);   // <= 1; 1 where this lane's m stays
                         l *= alpha;
-                        m = mn;
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
                     }
-                    float psum = 0.0f;
+                    m = mn;
+                    const float dsub = m - used;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        a0[r] = fast_exp2(a0[r] - m);
-                        a1[r] = fast_exp2(a1[r] - m);
-                        psum += a0[r] + a1[r];
+                        a0[r] -= dsub;
+                        a1[r] -= dsub;
                     }
-                    l += psum;
-                    // ---- O^T += V^T P^T, V^T fragments by transposing reads of row-major V
+                    // from the next scores on the MFMA subtracts m itself
+                    mf = fabsf(m) <= 1024.0f ? m : 0.0f;
+                    qaug = aug8<T>(ones3<T>(), pack_split3<T>(-mf));
+                }
+            };
+            // ---- part 2: P = exp2, rounded to T; row sums of the rounded values; O^T += V^T P^T
+            // with V^T fragments by transposing reads of row-major V
+            auto finish = [&](int step, f32x16 &a0, f32x16 &a1) {
+                const int kb = step * 64;
 #pragma unroll
-                    for (int ts = 0; ts < 4; ++ts) {
-                        v8 pf;
+                for (int r = 0; r < 16; ++r) {
+                    a0[r] = fast_exp2(a0[r]);
+                    a1[r] = fast_exp2(a1[r]);
+                }
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+                for (int ts = 0; ts < 4; ++ts) {
+                    v8 pf;
 #pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) {
-                            const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                            v8 va = zero8<T>();
-                            if (col < D) {
+                    for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+                    l = pair_sums<T>(pf, l);
 #pragma unroll
-                                for (int h2 = 0; h2 < 2; ++h2) {
-                                    const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
-                                    const unsigned char *ad = buf + R::OFF_V + R::swz(row, col >> 3) + (col & 7) * 2;
-                                    s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                        (s16x4 __attribute__((address_space(3))) *)ad);
-                                    v4 rv = __builtin_bit_cast(v4, rd);
-                                    va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
-                                }
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                        v8 va = zero8<T>();
+                        if (col < D) {
+#pragma unroll
+                            for (int h2 = 0; h2 < 2; ++h2) {
+                                const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                                const unsigned char *ad = buf + R::OFF_V + R::swz(row, col >> 3) + (col & 7) * 2;
+                                s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                    (s16x4 __attribute__((address_space(3))) *)ad);
+                                v4 rv = __builtin_bit_cast(v4, rd);
+                                va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
                             }
-                            oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
                         }
+                        oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
                     }
+                }
+            };
+            // (A second score set, so that the matrix core could form the scores of step s+1 under
+            // the softmax of step s, does not fit 256 registers next to the resident bias: the
+            // spilled form measured 153 us against 120 us at S = 512, N = 256, H = 8.)
+            f32x16 sa0, sa1;
+#pragma unroll
+            for (int step = 0; step < 4; ++step) {
+                EVO_TR(3 + step);
+                if (step < nsteps) {  // uniform
+                    const float used = mf;
+                    scores(step, sa0, sa1);
+                    settle(step, sa0, sa1, used);
+                    finish(step, sa0, sa1);
                 }
             }
 
+            EVO_TR(7);
             {   // the two lane groups hold the two halves of each query's sum
                 const unsigned u = __float_as_uint(l);
                 auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -318,7 +449,9 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     }
             }
         }
+        EVO_TR(8);
         stash(t + 1);   // into the other buffer, free since the barrier above
+        EVO_TR(9);
 #pragma unroll
         for (int ks = 0; ks < KSD; ++ks) qraw[ks] = qnext[ks];
     }
@@ -326,12 +459,12 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, bool HAS_BIAS>
+template <typename T, int D, int BIASK>
 static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
     typedef FwdRingGeo<D> R;
     static int cus = 0;
     static bool attr_set = false;
-    auto kern = mfma_fwd_ring<T, D, HAS_BIAS>;
+    auto kern = mfma_fwd_ring<T, D, BIASK>;
     if (!attr_set) {
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
@@ -355,7 +488,13 @@ static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) 
 
 template <typename T>
 static int fwdr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    return p.bias_dtype == EVO_NONE ? fwdr_launch<T, EVO_D, false>(p, e, st) : fwdr_launch<T, EVO_D, true>(p, e, st);
+    if (p.bias_dtype == EVO_NONE) return fwdr_launch<T, EVO_D, 0>(p, e, st);
+    // The 16-bit form reads the caller's bias rows in 16-byte pieces; where it applies it is the
+    // faster one (64 resident registers instead of 128, no spills).  Bit 0x400 of flags (not
+    // part of the public interface) selects the other form, for comparison.
+    const bool rows16 = p.bias_dtype == p.dtype && p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 &&
+                        p.bias_stride_b % 8 == 0 && p.bias_stride_h % 8 == 0 && p.bias_stride_row % 8 == 0;
+    return (rows16 && !(p.flags & 0x400)) ? fwdr_launch<T, EVO_D, 2>(p, e, st) : fwdr_launch<T, EVO_D, 1>(p, e, st);
 }
 
 // Largest N this kernel takes for the head dim (0: not built for it).
