@@ -250,7 +250,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             EVO_TR(1);
             lds_barrier();   // stage t is in LDS; stage t-1 and the last reduction are done with
             EVO_TR(2);
-            fetch(t + 1);
+            // The CU's load path takes a stage's 48 requests (D = 32) at 16 clocks each; the waves
+            // take turns (half now, half after the row's prologue) rather than all queue up behind
+            // it.  With few requests per wave there is nothing to gain.
+            const bool early = !(NBLK == 1 && IPW >= 4) || (wave & 1) == 0;
+            if (early) fetch(t + 1);
             EVO_TR(3);
             buf = lds + (t & 1) * R::BUF_BYTES;
 
@@ -296,6 +300,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 }
             }
 
+            if (!early) fetch(t + 1);
             EVO_TR(4);
             if (qact) {
 #pragma unroll
