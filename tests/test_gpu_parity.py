@@ -184,6 +184,10 @@ SMALL = [
     (1, 3, 250, 2, 64, "add", "q", "reference"),
     (1, 40, 256, 1, 32, "add", "q", "ds4sci"),
     (1, 9, 192, 2, 32, None, None, "reference"),
+    (2, 6, 256, 3, 32, "add", "q", "ds4sci"),          # per-head strides, bias per batch entry
+    (1, 5, 252, 2, 32, "bool", "q", "reference"),      # bias rows not 16-byte aligned: fp32 tiles
+    (1, 5, 256, 2, 16, "soft", torch.float32, "reference"),
+    (2, 3, 136, 2, 8, "add", "q", "reference"),
 ]
 
 
@@ -296,9 +300,10 @@ def test_non_contiguous_inputs_and_broadcast_operands(E):
     assert_close(got, ref, BF16_TOL, what="broadcast")
 
 
-def test_mask_edge_values(E):
+@pytest.mark.parametrize("N", [96, 256])      # one-workgroup-per-problem kernels / chunk-of-rows kernels
+def test_mask_edge_values(E, N):
     """-inf mask entries, a fully masked S row (bool and -1e9), all-kept, single kept key."""
-    B, S, N, H, D = 1, 4, 96, 2, 32
+    B, S, H, D = 1, 4, 2, 32
     Q, K, V, _, bias, dO = make_case(B, S, N, H, D, None, "q", torch.bfloat16)
     keep = torch.ones((B, S, 1, 1, N), dtype=torch.bool)
     keep[0, 0, 0, 0, 5:] = False           # keys 0..4 kept
@@ -317,9 +322,13 @@ def test_mask_edge_values(E):
         got = run_hip(E, Q, K, V, m, bias, dO)
         for n, t in got.items():
             assert torch.isfinite(t.float()).all(), (kind, n)
-        # the single kept key collects dV = sum of all 96 dO rows, |dV| ~ 20: allow one
+        # the single kept key collects dV = sum of all N dO rows, |dV| ~ 20..30: allow one
         # bf16 ulp of the entry on top of the absolute bound
-        assert_close(got, ref, BF16_TOL, what=f"mask {kind}", ulp_names=("dQ", "dK", "dV", "dBias"), ulps=2)
+        # At N = 256 five kept keys collect dK, dV from 256 queries each: sums of 256 products of
+        # probabilities rounded to bf16.  Eager evaluated in bf16 is 3.2e-2 away from the fp32
+        # values on this input; the bound follows it.
+        tol = BF16_TOL if N <= 96 else 3.5e-2
+        assert_close(got, ref, tol, what=f"mask {kind}", ulp_names=("dQ", "dK", "dV", "dBias"), ulps=2)
         Oh, Vh = eager.to_heads(got["O"].float().cpu()), eager.to_heads(V.float())
         assert (Oh[0, :, 2] - Vh[0, :, 2, 77:78]).abs().max() <= 1e-2       # single kept key: O = that V row
         assert (Oh[0, :, 1] - Vh[0, :, 1].mean(1, keepdim=True)).abs().max() <= 1e-2   # dead row: mean of V
