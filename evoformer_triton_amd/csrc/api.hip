@@ -65,13 +65,25 @@ static bool dq_ring_ok(const EvoAttnParams &p) {
 }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
-// writes one partial dBias tile.  Enough chunks to fill the chip, no more.
+// writes one partial dBias tile.  Enough chunks to fill the chip, no more.  The kernel that
+// walks over its chunk with one workgroup per CU (256 CUs) wants the workgroups to come in
+// whole rounds: among the chunk counts that give one to four rounds it takes the one that
+// leaves the fewest CUs idle in the last round (ties: the fewest chunks).
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t NT = (p.N + 31) / 32;
-    const bool ring = dq_ring_ok(p);   // 64 query rows and 8 waves per workgroup, one workgroup per CU
+    const bool ring = dq_ring_ok(p);
     const int64_t base = (ring ? (NT + 1) / 2 : NT) * p.B * p.H;
-    const int64_t target = ring ? 512 : 1024;
-    int64_t want = (target + base - 1) / base;
+    int64_t want = (1024 + base - 1) / base;
+    if (ring) {
+        constexpr int64_t CUS = 256;
+        const int64_t lo = (CUS + base - 1) / base, hi = (4 * CUS + base - 1) / base;
+        double best = -1.0;
+        for (int64_t n = lo; n <= hi; ++n) {
+            const int64_t wgs = base * n, rounds = (wgs + CUS - 1) / CUS;
+            const double eff = (double)wgs / (double)(rounds * CUS);
+            if (eff > best + 1e-9) { best = eff; want = n; }
+        }
+    }
     if (want < 1) want = 1;
     if (want > p.S) want = p.S;
     *chunk = (int)((p.S + want - 1) / want);
