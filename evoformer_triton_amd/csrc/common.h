@@ -103,6 +103,14 @@ __device__ __forceinline__ bool ds_blocked(const EvoAttnParams &p, float shift) 
     return p.mask_kind == EVO_MASK_BOOL && shift != 0.0f;
 }
 
+// An int that every lane of the wave reads from the same address, written by an earlier
+// kernel: through the constant address space, i.e. a scalar load.  As an ordinary load it
+// would be a vector load, and waiting for it would also wait for every older vector store
+// of the wave (vector memory operations complete in order).
+__device__ __forceinline__ int uniform_load(const int *ptr) {
+    return *(const __attribute__((address_space(4))) int *)(ptr);
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 
 __device__ __forceinline__ float wave_max(float v) {

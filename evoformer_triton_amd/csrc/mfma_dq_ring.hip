@@ -49,7 +49,8 @@ struct RingGeo {
     static constexpr int OFF_Q = OFF_A + A_BYTES;
     static constexpr int OFF_G = OFF_Q + Q_BYTES;
     static constexpr int OFF_O = OFF_G + Q_BYTES;
-    static constexpr int STAGE_BYTES = OFF_O + Q_BYTES;
+    static constexpr int OFF_L = OFF_O + Q_BYTES;                   // log-sum-exp of the QR query rows, fp32
+    static constexpr int STAGE_BYTES = OFF_L + QR * 4;
     static constexpr int RED_BYTES = 8 * 32 * RP * 4;
     static constexpr int BUF_BYTES = ((STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES) + 1023) / 1024 * 1024;
     static constexpr int LDS_BYTES = 2 * BUF_BYTES;
@@ -148,6 +149,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // assigns to some chunk of some row.
     constexpr int IPW = (R::I_ALL + 7) / 8;   // most pieces one wave moves per stage
     u32x4 stg[IPW];
+    float lse_stg = 0.0f;
     // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
     // Where piece n of key block blk comes from and goes to: a base that every lane shares for
@@ -204,6 +206,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             const Piece d = NBLK == 1 ? fixed[i] : describe(min(wave + 8 * i, ninst - 1), blk);
             stg[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
         }
+        // the log-sum-exp of the slab's rows travels the same way (one value per lane; every
+        // wave asks, wave 0 stores): a load whose result is carried into the next row's
+        // prologue in a register would make that prologue wait for everything requested here
+        lse_stg = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
     };
     auto stash = [&](int t) {
         const int blk = t % NBLK;
@@ -217,12 +223,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
             }
         }
+        if (wave == 0 && blk == 0 && t < T_total) *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
     };
 
     fetch(0);
     stash(0);
-    float lse_nxt = 0.0f;
-    if (T_total > 0) lse_nxt = p.lse[(int64_t)(bh * (unsigned)p.S + s_begin) * p.N + qrow];
 
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
@@ -233,7 +238,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         pr.b = b; pr.h = h; pr.s = s;
         pr.base = base0 + (int64_t)(s - s_begin) * p.stride_s;
         pr.row0 = (int64_t)pid * p.N;
-        const bool dead = e.dead[b * p.S + s] != 0;
+        const bool dead = uniform_load(e.dead + b * p.S + s) != 0;
         const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
 
         v8 qf[KS], gf[KS], qlo[KSD];
@@ -260,8 +265,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
             if (blk == 0) {
                 // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
-                const float lse2 = lse_nxt * kLog2e;
-                if (s + 1 < s_end) lse_nxt = p.lse[(int64_t)(pid + 1) * p.N + qrow];
+                const float lse2 = *reinterpret_cast<const float *>(buf + R::OFF_L + (qi * 32 + li) * 4) * kLog2e;
                 float dpart = 0.0f;
 #pragma unroll
                 for (int ks = 0; ks < KSD; ++ks) qlo[ks] = zero8<T>();

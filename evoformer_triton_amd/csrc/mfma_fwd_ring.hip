@@ -251,7 +251,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     for (int t = 0; t < nrows; ++t) {
         const int s = s_begin + t;
         const unsigned pid = bh * (unsigned)p.S + s;
-        const bool dead = e.dead[b * p.S + s] != 0;
+        const bool dead = uniform_load(e.dead + b * p.S + s) != 0;
         EVO_TR(0);
         lds_barrier_f();   // the stage of this row is in LDS; everybody is done with the row before
         EVO_TR(1);
@@ -260,6 +260,11 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         EVO_TR(2);
         const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 
+        // m: the maximum the probabilities are relative to; mf: what the mask k-step currently
+        // subtracts inside the MFMA (m, or 0 while m is not yet known or too large to be
+        // carried in three 16-bit columns next to scores of order one)
+        float m = 0.0f, mf = 0.0f, l = 0.0f;
+        f32x16 oacc[DT];
         if (qact) {
             v8 qf[KSD], qlo[KSD];
             const float cq = dead ? 0.0f : cscale;
@@ -269,12 +274,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 qlo[ks] = zero8<T>();
                 if (2 * ks + g < C) scaled_hilo8<T>(qraw[ks], cq, qf[ks], qlo[ks]);
             }
-            // m: the maximum the probabilities are relative to; mf: what the mask k-step
-            // currently subtracts inside the MFMA (m, or 0 while m is not yet known or too
-            // large to be carried in three 16-bit columns next to scores of order one)
-            float m = 0.0f, mf = 0.0f, l = 0.0f;
             v8 qaug = aug8<T>(ones3<T>(), uint2{0u, 0u});   // ones x mask columns, -mf x ones
-            f32x16 oacc[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -427,6 +427,14 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 }
             }
 
+        }
+        // The next stage goes into the other buffer, free since the barrier above.  This comes
+        // before the row's own stores: what waits for the staged loads must not have the
+        // stores in front of it (vector memory operations complete in order).
+        EVO_TR(8);
+        stash(t + 1);
+        EVO_TR(9);
+        if (qact) {
             EVO_TR(7);
             {   // the two lane groups hold the two halves of each query's sum
                 const unsigned u = __float_as_uint(l);
@@ -439,19 +447,9 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 T *O = (T *)p.o + base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
                 if (g == 0) p.lse[(int64_t)pid * p.N + q] = (m + __log2f(l)) * kLn2;
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) {
-                        const int d0 = dt * 32 + 8 * rr + 4 * g;
-                        if (d0 < D)
-                            store4<T>(O + d0, oacc[dt][4 * rr] * inv, oacc[dt][4 * rr + 1] * inv,
-                                      oacc[dt][4 * rr + 2] * inv, oacc[dt][4 * rr + 3] * inv);
-                    }
+                for (int dt = 0; dt < DT; ++dt) store_row_tile<T>(O, dt * 32, D, oacc[dt], inv, g);
             }
         }
-        EVO_TR(8);
-        stash(t + 1);   // into the other buffer, free since the barrier above
-        EVO_TR(9);
 #pragma unroll
         for (int ks = 0; ks < KSD; ++ks) qraw[ks] = qnext[ks];
     }
