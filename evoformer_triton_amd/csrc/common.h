@@ -196,6 +196,35 @@ __device__ __forceinline__ void scaled_hilo8(typename Mfma<T>::v8 raw, float c, 
     }
 }
 
+// acc + <a, b> over 8 elements of T, the products and sums in fp32 (`v_dot2c_f32_{bf16,f16}`:
+// two elements per instruction and no conversions).
+template <typename T>
+__device__ __forceinline__ float dot8(typename Mfma<T>::v8 a, typename Mfma<T>::v8 b, float acc);
+template <>
+__device__ __forceinline__ float dot8<bf16_t>(bf16x8 a, bf16x8 b, float acc) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bf2 x, y;
+        x[0] = a[2 * i]; x[1] = a[2 * i + 1];
+        y[0] = b[2 * i]; y[1] = b[2 * i + 1];
+        acc = __builtin_amdgcn_fdot2_f32_bf16(x, y, acc, false);
+    }
+    return acc;
+}
+template <>
+__device__ __forceinline__ float dot8<f16_t>(f16x8 a, f16x8 b, float acc) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        h2 x, y;
+        x[0] = a[2 * i]; x[1] = a[2 * i + 1];
+        y[0] = b[2 * i]; y[1] = b[2 * i + 1];
+        acc = __builtin_amdgcn_fdot2(x, y, acc, false);
+    }
+    return acc;
+}
+
 // (hi, mid, lo, 0) of split3 packed into 8 bytes.
 template <typename T>
 __device__ __forceinline__ uint2 pack_split3(float m) {

@@ -130,8 +130,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
                 gf[ks] = ld8(Gd + (int64_t)qrow * sn + d0);
                 v8 oraw = ld8(O + (int64_t)qrow * sn + d0);
                 if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) dpart = fmaf((float)gf[ks][i], (float)oraw[i], dpart);
+                dpart = dot8<T>(gf[ks], oraw, dpart);
             }
         }
         const float dl = dpart + __shfl_xor(dpart, 32);

@@ -52,8 +52,12 @@ struct RingGeo {
     static constexpr int OFF_L = OFF_O + Q_BYTES;                   // log-sum-exp of the QR query rows, fp32
     static constexpr int STAGE_BYTES = OFF_L + QR * 4;
     static constexpr int RED_BYTES = 8 * 32 * RP * 4;
-    static constexpr int BUF_BYTES = ((STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES) + 1023) / 1024 * 1024;
-    static constexpr int LDS_BYTES = 2 * BUF_BYTES;
+    static constexpr int STAGE_1K = (STAGE_BYTES + 1023) / 1024 * 1024;
+    // The partial dQ tiles get LDS of their own where 160 KB allow it; otherwise they lie in the
+    // buffer of the stage just consumed.
+    static constexpr bool OWN_RED = 2 * STAGE_1K + RED_BYTES <= 160 * 1024;
+    static constexpr int BUF_BYTES = OWN_RED ? STAGE_1K : ((STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES) + 1023) / 1024 * 1024;
+    static constexpr int LDS_BYTES = OWN_RED ? 2 * BUF_BYTES + RED_BYTES : 2 * BUF_BYTES;
     // 1 KB pieces (64 lanes x 16 bytes) per segment of a stage
     static constexpr int I_K = K_BYTES / 1024, I_A = A_BYTES / 1024, I_Q = Q_BYTES / 1024;
     static constexpr int I_KVA = 2 * I_K + I_A;
@@ -107,14 +111,6 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     const int64_t sn = p.stride_n;
     const bool want_dbias = e.dbias_part != nullptr && p.dbias != nullptr;
     const float cs = p.scale * kLog2e;
-
-    // identity slices in fp16: A[m][8g+i] = 1 where m is the key row that register 8ts+i of
-    // an accumulator tile holds for lane group g
-    f16x8 idf[2];
-#pragma unroll
-    for (int ts = 0; ts < 2; ++ts)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) idf[ts][i] = (f16_t)(li == crow(8 * ts + i, g) ? 1.0f : 0.0f);
 
     f32x16 dbacc[NSLOT];
 #pragma unroll
@@ -226,6 +222,31 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         if (wave == 0 && blk == 0 && t < T_total) *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
     };
 
+    // The four partial dQ^T tiles of a query tile (one per wave, fp32, in the buffer of the
+    // stage they came from) summed, scaled and stored as row `base` of dQ.
+    auto sum_store = [&](const float *red, int64_t base) {
+        T *dQ = (T *)p.dq + base;
+        for (int it = tid; it < 64 * (D / 4); it += 512) {
+            const int q = it / (D / 4), d4 = (it % (D / 4)) * 4;
+            const int w0 = (q >> 5) * 4, ql = q & 31;
+            f32x4 sum = *reinterpret_cast<const f32x4 *>(&red[(w0 * 32 + ql) * RP + d4]);
+#pragma unroll
+            for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
+            if (qbase + q < p.N)
+                store4<T>(dQ + (int64_t)(qbase + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
+                          sum[3] * p.scale);
+        }
+    };
+    // With one key block per row the sum of a row's partials waits until the next row's stage
+    // barrier has been passed (two barriers per row instead of three): nobody writes where the
+    // partials lie before the barrier that follows the next row's tiles.
+    constexpr bool DEFER = NBLK == 1;
+    // With the partials out of the stage buffers, the buffer of the next stage is free from
+    // the stage barrier on: a wave whose requests went out at the top of the row writes what
+    // they returned between its tiles, while other waves compute, rather than all at the end.
+    constexpr bool MID = DEFER && R::OWN_RED && TPW >= 2;
+    auto red_of = [&](int stage) { return (float *)(lds + (R::OWN_RED ? 2 * R::BUF_BYTES : (stage & 1) * R::BUF_BYTES)); };
+
     fetch(0);
     stash(0);
 
@@ -262,6 +283,8 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             if (early) fetch(t + 1);
             EVO_TR(3);
             buf = lds + (t & 1) * R::BUF_BYTES;
+            if (DEFER && s > s_begin)
+                sum_store(red_of(t - 1), pr.base - p.stride_s);
 
             if (blk == 0) {
                 // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
@@ -280,8 +303,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         gf[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_G + o);
                         const v8 oraw = *reinterpret_cast<const v8 *>(buf + R::OFF_O + o);
                         if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) dpart = fmaf((float)gf[ks][i], (float)oraw[i], dpart);
+                        dpart = dot8<T>(gf[ks], oraw, dpart);
                     }
                 }
                 float dl;
@@ -306,12 +328,13 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
             if (!early) fetch(t + 1);
             EVO_TR(4);
-            if (qact) {
+            {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
                     const int tb = jj * 4 + kq;          // tile inside the stage
                     const int kt = blk * TPB + tb;
-                    if (kt < NT) {  // wave-uniform
+                    if (MID && early && jj == TPW - 1) stash(t + 1);
+                    if (qact && kt < NT) {  // wave-uniform
                         const int slot = blk * TPW + jj;
                         v8 ka[KS], va[KS];
 #pragma unroll
@@ -347,16 +370,15 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         float ds[16];
 #pragma unroll
                         for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(acc[r]) * dp[r];
+                        if (want_dbias) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) dbacc[slot][r] += ds[r];
+                        }
 #pragma unroll
                         for (int ts = 0; ts < 2; ++ts) {
                             v8 dsf;
-                            f16x8 dsh;
 #pragma unroll
-                            for (int i = 0; i < 8; ++i) {
-                                dsf[i] = (T)ds[8 * ts + i];
-                                dsh[i] = (f16_t)ds[8 * ts + i];
-                            }
-                            if (want_dbias) dbacc[slot] = Mfma<f16_t>::mma(idf[ts], dsh, dbacc[slot]);
+                            for (int i = 0; i < 8; ++i) dsf[i] = (T)ds[8 * ts + i];
 #pragma unroll
                             for (int dt = 0; dt < DT; ++dt) {
                                 // K^T fragment: row d = dt*32 + li, the 8 keys the dS^T registers hold
@@ -379,7 +401,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     }
                 }
             }
-            stash(t + 1);   // into the other buffer, free since the barrier above
+            if (!DEFER || (MID && !early)) stash(t + 1);   // into the other buffer, free since the barrier above
         }
 
         // Partial dQ^T of this wave: lane = query li, register r = dim dt*32 + crow(r, g).  The
@@ -387,7 +409,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         EVO_TR(5);
         lds_barrier();
         EVO_TR(6);
-        float *red = (float *)(lds + ((t - 1) & 1) * R::BUF_BYTES);
+        float *red = red_of(t - 1);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -398,22 +420,22 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 *reinterpret_cast<f32x4 *>(&red[(wave * 32 + li) * RP + dt * 32 + 8 * rr + 4 * g]) = v;
             }
         EVO_TR(7);
-        lds_barrier();
-        EVO_TR(8);
-        T *dQ = (T *)p.dq + pr.base;
-        for (int it = tid; it < 64 * (D / 4); it += 512) {
-            const int q = it / (D / 4), d4 = (it % (D / 4)) * 4;
-            const int w0 = (q >> 5) * 4, ql = q & 31;
-            f32x4 sum = *reinterpret_cast<const f32x4 *>(&red[(w0 * 32 + ql) * RP + d4]);
-#pragma unroll
-            for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
-            if (qbase + q < p.N)
-                store4<T>(dQ + (int64_t)(qbase + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
-                          sum[3] * p.scale);
+        if (DEFER) {
+            // the other buffer held the last row's partials; everyone has summed them by now
+            if (!MID) stash(t);
+            EVO_TR(8);
+        } else {
+            lds_barrier();
+            EVO_TR(8);
+            sum_store(red, pr.base);
         }
         EVO_TR(9);
         // the barrier at the top of the next stage keeps the next request for this buffer
         // behind these reads
+    }
+    if (DEFER && s_end > s_begin) {
+        lds_barrier();
+        sum_store(red_of(t - 1), base0 + (int64_t)(s_end - 1 - s_begin) * p.stride_s);
     }
 
     if (want_dbias && qact && q0 + li < p.N) {

@@ -69,32 +69,11 @@ __device__ __forceinline__ void lds_barrier_f() { asm volatile("s_waitcnt lgkmcn
 
 // acc + the sum of the eight 16-bit values of x, two per instruction.
 template <typename T>
-__device__ __forceinline__ float pair_sums(typename Mfma<T>::v8 x, float acc);
-template <>
-__device__ __forceinline__ float pair_sums<bf16_t>(bf16x8 x, float acc) {
-    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-    bf2 one;
-    one[0] = one[1] = (__bf16)1.0f;
+__device__ __forceinline__ float pair_sums(typename Mfma<T>::v8 x, float acc) {
+    typename Mfma<T>::v8 one;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        bf2 v;
-        v[0] = x[2 * i]; v[1] = x[2 * i + 1];
-        acc = __builtin_amdgcn_fdot2_f32_bf16(v, one, acc, false);
-    }
-    return acc;
-}
-template <>
-__device__ __forceinline__ float pair_sums<f16_t>(f16x8 x, float acc) {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2 one;
-    one[0] = one[1] = (_Float16)1.0f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        h2 v;
-        v[0] = x[2 * i]; v[1] = x[2 * i + 1];
-        acc = __builtin_amdgcn_fdot2(v, one, acc, false);
-    }
-    return acc;
+    for (int i = 0; i < 8; ++i) one[i] = (T)1.0f;
+    return dot8<T>(x, one, acc);
 }
 
 // BIASK: 0 no bias, 1 fp32 tiles (x log2(e), accumulator order) as C operands, 2 the caller's 16-bit rows through the identity
