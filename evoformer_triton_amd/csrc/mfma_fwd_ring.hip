@@ -125,20 +125,12 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
             }
         }
     }
-    // (identity x log2(e)) as A operands, hi and lo parts: row = key li of the tile, column 16 ks + 8 g + i
-    v8 idh[2], idl[2];
-    {
-        const T chi = (T)kLog2e;
-        const T clo = (T)(kLog2e - (float)chi);
+    // the identity as A operands: row = key li of the tile, column 16 ks + 8 g + i
+    v8 idh[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const bool on = li == 16 * ks + 8 * g + i;
-                idh[ks][i] = on ? chi : (T)0.0f;
-                idl[ks][i] = on ? clo : (T)0.0f;
-            }
-    }
+        for (int i = 0; i < 8; ++i) idh[ks][i] = (T)(li == 16 * ks + 8 * g + i ? 1.0f : 0.0f);
     if (BIASK == 2) {
         const int bb = e.bias_batches > 1 ? b : 0;
         const T *brow = (const T *)p.bias + (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h +
@@ -267,14 +259,17 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     f32x16 z;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+                    // the bias tile itself through the matrix core (exact: one product per
+                    // element), then into log2 units in fp32; a scaled identity would need a hi
+                    // and a lo part of the constant, twice the MFMAs
                     a0 = Mfma<T>::mma(idh[0], bres[4 * step], z);
                     a1 = Mfma<T>::mma(idh[0], bres[4 * step + 2], z);
-                    a0 = Mfma<T>::mma(idl[0], bres[4 * step], a0);
-                    a1 = Mfma<T>::mma(idl[0], bres[4 * step + 2], a1);
                     a0 = Mfma<T>::mma(idh[1], bres[4 * step + 1], a0);
                     a1 = Mfma<T>::mma(idh[1], bres[4 * step + 3], a1);
-                    a0 = Mfma<T>::mma(idl[1], bres[4 * step + 1], a0);
-                    a1 = Mfma<T>::mma(idl[1], bres[4 * step + 3], a1);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) a0[r] *= kLog2e;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) a1[r] *= kLog2e;
                     started = true;
                 }
 #pragma unroll
