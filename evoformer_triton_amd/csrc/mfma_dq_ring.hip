@@ -193,34 +193,41 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     }
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
-    auto fetch = [&](int t) {
+    // pieces [i0, i1) of stage t; the last piece takes the log-sum-exp along
+    auto fetch_part = [&](int t, int i0, int i1) {
         t = min(t, T_total - 1);
         const int row = t / NBLK, blk = t % NBLK;
         const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
+            if (i < i0 || i >= i1) continue;
             const Piece d = NBLK == 1 ? fixed[i] : describe(min(wave + 8 * i, ninst - 1), blk);
             stg[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
         }
         // the log-sum-exp of the slab's rows travels the same way (one value per lane; every
         // wave asks, wave 0 stores): a load whose result is carried into the next row's
         // prologue in a register would make that prologue wait for everything requested here
-        lse_stg = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
+        if (i1 >= IPW) lse_stg = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
     };
-    auto stash = [&](int t) {
+    auto fetch = [&](int t) { fetch_part(t, 0, IPW); };
+    constexpr int SPLIT = IPW / 2;   // pieces asked for at the top of a row; the rest after its prologue
+    auto stash_part = [&](int t, int i0, int i1) {
         const int blk = t % NBLK;
         const int ninst = t >= T_total ? 0 : blk == 0 ? R::I_ALL : R::I_KVA;
         unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
+            if (i < i0 || i >= i1) continue;
             const int n = wave + 8 * i;
             if (n < ninst) {
                 const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
                 *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
             }
         }
-        if (wave == 0 && blk == 0 && t < T_total) *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
+        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total)
+            *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
     };
+    auto stash = [&](int t) { stash_part(t, 0, IPW); };
 
     // The four partial dQ^T tiles of a query tile (one per wave, fp32, in the buffer of the
     // stage they came from) summed, scaled and stored as row `base` of dQ.
@@ -242,8 +249,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // partials lie before the barrier that follows the next row's tiles.
     constexpr bool DEFER = NBLK == 1;
     // With the partials out of the stage buffers, the buffer of the next stage is free from
-    // the stage barrier on: a wave whose requests went out at the top of the row writes what
-    // they returned between its tiles, while other waves compute, rather than all at the end.
+    // the stage barrier on: every wave asks for half of its pieces at the top of the row and
+    // writes them to LDS between its two tiles, while other waves compute; the other half it
+    // asks for after the row's prologue and writes after the tiles.
     constexpr bool MID = DEFER && R::OWN_RED && TPW >= 2;
     auto red_of = [&](int stage) { return (float *)(lds + (R::OWN_RED ? 2 * R::BUF_BYTES : (stage & 1) * R::BUF_BYTES)); };
 
@@ -276,11 +284,13 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             EVO_TR(1);
             lds_barrier();   // stage t is in LDS; stage t-1 and the last reduction are done with
             EVO_TR(2);
-            // The CU's load path takes a stage's 48 requests (D = 32) at 16 clocks each; the waves
-            // take turns (half now, half after the row's prologue) rather than all queue up behind
-            // it.  With few requests per wave there is nothing to gain.
+            // The CU's load path takes a stage's 48 requests (D = 32) at 16 clocks each: half of
+            // them go out now and half after the row's prologue rather than all queue up behind
+            // it (where the staging writes cannot be split, the waves take turns instead).  With
+            // few requests per wave there is nothing to gain.
             const bool early = !(NBLK == 1 && IPW >= 4) || (wave & 1) == 0;
-            if (early) fetch(t + 1);
+            if (MID) fetch_part(t + 1, 0, SPLIT);
+            else if (early) fetch(t + 1);
             EVO_TR(3);
             buf = lds + (t & 1) * R::BUF_BYTES;
             if (DEFER && s > s_begin)
@@ -326,14 +336,15 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 }
             }
 
-            if (!early) fetch(t + 1);
+            if (MID) fetch_part(t + 1, SPLIT, IPW);
+            else if (!early) fetch(t + 1);
             EVO_TR(4);
             {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
                     const int tb = jj * 4 + kq;          // tile inside the stage
                     const int kt = blk * TPB + tb;
-                    if (MID && early && jj == TPW - 1) stash(t + 1);
+                    if (MID && jj == TPW - 1) stash_part(t + 1, 0, SPLIT);
                     if (qact && kt < NT) {  // wave-uniform
                         const int slot = blk * TPW + jj;
                         v8 ka[KS], va[KS];
@@ -401,7 +412,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     }
                 }
             }
-            if (!DEFER || (MID && !early)) stash(t + 1);   // into the other buffer, free since the barrier above
+            // into the other buffer, free since the barrier above
+            if (MID) stash_part(t + 1, SPLIT, IPW);
+            else if (!DEFER) stash(t + 1);
         }
 
         // Partial dQ^T of this wave: lane = query li, register r = dim dt*32 + crow(r, g).  The

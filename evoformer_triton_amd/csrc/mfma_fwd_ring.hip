@@ -190,11 +190,13 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     }
     // Loads are unconditional (the row past the end repeats the last row) so that the
     // staging registers stay registers.
-    auto fetch = [&](int t) {
+    auto fetch_piece = [&](int t, int i) {
         t = min(t, nrows - 1);
+        stg[i] = *reinterpret_cast<const u32x4 *>(pc[i].base + t * pc[i].row_step + pc[i].lane_off);
+    };
+    auto fetch = [&](int t) {
 #pragma unroll
-        for (int i = 0; i < IPW; ++i)
-            stg[i] = *reinterpret_cast<const u32x4 *>(pc[i].base + t * pc[i].row_step + pc[i].lane_off);
+        for (int i = 0; i < IPW; ++i) fetch_piece(t, i);
     };
     auto stash = [&](int t) {
         if (t >= nrows) return;
@@ -226,8 +228,6 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         EVO_TR(0);
         lds_barrier_f();   // the stage of this row is in LDS; everybody is done with the row before
         EVO_TR(1);
-        fetch(t + 1);
-        fetch_q(t + 1, qnext);
         EVO_TR(2);
         const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
 
@@ -361,6 +361,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     a0[r] = fast_exp2(a0[r]);
                     a1[r] = fast_exp2(a1[r]);
                 }
+                if (step == 2) EVO_TR(12);
 #pragma unroll
                 for (int ts = 0; ts < 4; ++ts) {
                     v8 pf;
@@ -393,14 +394,31 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 #pragma unroll
             for (int step = 0; step < 4; ++step) {
                 EVO_TR(3 + step);
+                {
+                    // The next row's requests go out a few per step rather than all after the
+                    // barrier: eight waves asking at once queue up behind the CU's load path
+                    // (16 clocks per request), and the last in line start their row late.
+                    constexpr int PPS = (IPW + 2) / 3;
+#pragma unroll
+                    for (int i = step * PPS; i < (step + 1) * PPS && i < IPW; ++i)
+                        if (step < 3) fetch_piece(t + 1, i);
+                    if (step == 2) fetch_q(t + 1, qnext);
+                }
                 if (step < nsteps) {  // uniform
                     const float used = mf;
                     scores(step, sa0, sa1);
+                    if (step == 2) EVO_TR(10);
                     settle(step, sa0, sa1, used);
+                    if (step == 2) EVO_TR(11);
                     finish(step, sa0, sa1);
+                    if (step == 2) EVO_TR(13);
                 }
             }
 
+        }
+        else {
+            fetch(t + 1);
+            fetch_q(t + 1, qnext);
         }
         // The next stage goes into the other buffer, free since the barrier above.  This comes
         // before the row's own stores: what waits for the staged loads must not have the
