@@ -239,6 +239,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         if (qact) {
             v8 qf[KSD], qlo[KSD];
             const float cq = dead ? 0.0f : cscale;
+            const float bscale = dead ? 0.0f : kLog2e;
 #pragma unroll
             for (int ks = 0; ks < KSD; ++ks) {
                 qf[ks] = zero8<T>();
@@ -255,7 +256,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
             auto scores = [&](int step, f32x16 &a0, f32x16 &a1) {
                 const int kb = step * 64;
                 bool started = false;
-                if (BIASK == 2 && !dead) {  // uniform
+                if (BIASK == 2) {
                     f32x16 z;
 #pragma unroll
                     for (int r = 0; r < 16; ++r) z[r] = 0.0f;
@@ -266,10 +267,11 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     a1 = Mfma<T>::mma(idh[0], bres[4 * step + 2], z);
                     a0 = Mfma<T>::mma(idh[1], bres[4 * step + 1], a0);
                     a1 = Mfma<T>::mma(idh[1], bres[4 * step + 3], a1);
+                    // (a row with every key masked takes no bias: the factor is 0 there)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) a0[r] *= kLog2e;
+                    for (int r = 0; r < 16; ++r) a0[r] *= bscale;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) a1[r] *= kLog2e;
+                    for (int r = 0; r < 16; ++r) a1[r] *= bscale;
                     started = true;
                 }
 #pragma unroll
@@ -352,22 +354,27 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     qaug = aug8<T>(ones3<T>(), pack_split3<T>(-mf));
                 }
             };
-            // ---- part 2: P = exp2, rounded to T; row sums of the rounded values; O^T += V^T P^T
-            // with V^T fragments by transposing reads of row-major V
-            auto finish = [&](int step, f32x16 &a0, f32x16 &a1) {
-                const int kb = step * 64;
+            // ---- part 2: P = exp2, rounded to T, and this lane's sum of the rounded values
+            auto probs = [&](f32x16 &a0, f32x16 &a1, v8 (&pf)[4], float &ls) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     a0[r] = fast_exp2(a0[r]);
                     a1[r] = fast_exp2(a1[r]);
                 }
-                if (step == 2) EVO_TR(12);
+                ls = 0.0f;
 #pragma unroll
                 for (int ts = 0; ts < 4; ++ts) {
-                    v8 pf;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
-                    l = pair_sums<T>(pf, l);
+                    for (int i = 0; i < 8; ++i) pf[ts][i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+                    ls = pair_sums<T>(pf[ts], ls);
+                }
+            };
+            // ---- part 3: O^T += V^T P^T with V^T fragments by transposing reads of row-major V
+            auto weigh = [&](int step, const v8 (&pf)[4], float ls) {
+                const int kb = step * 64;
+                l += ls;
+#pragma unroll
+                for (int ts = 0; ts < 4; ++ts) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
                         const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -383,7 +390,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                                 va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
                             }
                         }
-                        oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
+                        oacc[dt] = Mfma<T>::mma(va, pf[ts], oacc[dt]);
                     }
                 }
             };
@@ -408,9 +415,26 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     const float used = mf;
                     scores(step, sa0, sa1);
                     if (step == 2) EVO_TR(10);
-                    settle(step, sa0, sa1, used);
+                    v8 pf[4];
+                    float ls;
+                    // After the first step the scores come out of the MFMA relative to m already
+                    // (where m fits the mask columns): the step skips the search for its maximum
+                    // and looks at the sums instead.  A lane sum beyond 2^13 (or not a number)
+                    // means some score stands far above m: the step is then redone the long way.
+                    bool settled = step != 0 && !__any(m != used);
+                    if (settled) {
+                        probs(sa0, sa1, pf, ls);
+                        if (__any(!(ls <= 8192.0f))) {
+                            settled = false;
+                            scores(step, sa0, sa1);
+                        }
+                    }
+                    if (!settled) {
+                        settle(step, sa0, sa1, used);
+                        probs(sa0, sa1, pf, ls);
+                    }
                     if (step == 2) EVO_TR(11);
-                    finish(step, sa0, sa1);
+                    weigh(step, pf, ls);
                     if (step == 2) EVO_TR(13);
                 }
             }

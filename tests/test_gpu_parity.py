@@ -338,6 +338,40 @@ def test_mask_edge_values(E, N):
             assert got["dBias"][..., dead_cols].abs().max().item() == 0
 
 
+@pytest.mark.parametrize("where", ["ramp", "late_bias", "mask_front"])
+def test_forward_maximum_found_in_a_later_key_block(E, where):
+    """The chunk-of-rows forward takes the first 64 keys' maximum as the reference point of a
+    row's probabilities and redoes a later block the long way when its scores stand far above
+    it: scores that grow by tens of units from one block of 64 keys to the next (the bias is
+    exact in 16 bits, so the comparison stays sharp), steadily or in jumps, or because the mask
+    removes the first blocks."""
+    B, S, N, H, D = 1, 6, 256, 2, 32
+    Q, K, V, _, bias, dO = make_case(B, S, N, H, D, None, "q", torch.bfloat16, seed=11)
+    m = None
+    if where == "ramp":
+        bias = (bias.float() + 0.1 * torch.arange(N, dtype=torch.float32)).to(torch.bfloat16)   # +6.4 per block
+    elif where == "late_bias":
+        bias = bias.clone()
+        bias[..., 64:128] += 20.0
+        bias[..., 128:192] += 45.0
+        bias[..., 192:] += 90.0
+    else:
+        keep = torch.ones((B, S, 1, 1, N), dtype=torch.bool)
+        keep[:, ::2, :, :, :130] = False      # every other row starts at key 130
+        m = keep
+        bias = bias.clone()
+        bias[..., 130:] += 30.0
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
+    got = run_hip(E, Q, K, V, m, bias, dO)
+    for n, t in got.items():
+        assert torch.isfinite(t.float()).all(), (where, n)
+    # The ramp puts nearly all of every row's weight on the last dozen keys, whose dK and dV
+    # collect 256 products of probabilities rounded to bf16 (eager evaluated in bf16 is 0.19
+    # away from the fp32 values on this input, the one-workgroup-per-problem kernels 0.025).
+    tol = 3e-2 if where == "ramp" else BF16_TOL
+    assert_close(got, ref, tol, what=where, ulp_names=("dQ", "dK", "dV", "dBias"), ulps=2)
+
+
 def test_checkpoint_recompute_and_no_grad(E):
     from torch.utils.checkpoint import checkpoint
     Q, K, V, m, bias, dO = make_case(1, 3, 64, 2, 32, "bool", "q", torch.bfloat16)
