@@ -61,7 +61,7 @@ static int bias_vec_ok(const EvoAttnParams &p) {
 
 // The dQ kernel that double-buffers its operands in LDS takes rows of limited length.
 static bool dq_ring_ok(const EvoAttnParams &p) {
-    return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N <= mfma_dqr_max_n(p.D);
+    return !(p.flags & EVO_FLAG_PER_PROBLEM) && mfma_dqr_qrows(p.D, p.N) > 0;
 }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
@@ -72,7 +72,8 @@ static bool dq_ring_ok(const EvoAttnParams &p) {
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t NT = (p.N + 31) / 32;
     const bool ring = dq_ring_ok(p);
-    const int64_t base = (ring ? (NT + 1) / 2 : NT) * p.B * p.H;
+    // workgroups per chunk: one per slab of query rows and head
+    const int64_t base = (ring ? (p.N + mfma_dqr_qrows(p.D, p.N) - 1) / mfma_dqr_qrows(p.D, p.N) : NT) * p.B * p.H;
     int64_t want = (1024 + base - 1) / base;
     if (ring) {
         constexpr int64_t CUS = 256;

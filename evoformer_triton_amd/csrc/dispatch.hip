@@ -10,7 +10,7 @@ namespace evo {
     int mfma_fwdr_max_n_d##D();                                                              \
     int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
     int launch_mfma_dqr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
-    int mfma_dqr_max_n_d##D();                                                               \
+    int mfma_dqr_qrows_d##D(int);                                                            \
     int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
 EVO_DECL(16)
@@ -45,12 +45,12 @@ int mfma_fwdr_max_n(int D) {
     return 0;
 }
 
-int mfma_dqr_max_n(int D) {
+int mfma_dqr_qrows(int D, int N) {
     switch (D) {
-        case 8: return mfma_dqr_max_n_d8();
-        case 16: return mfma_dqr_max_n_d16();
-        case 32: return mfma_dqr_max_n_d32();
-        case 64: return mfma_dqr_max_n_d64();
+        case 8: return mfma_dqr_qrows_d8(N);
+        case 16: return mfma_dqr_qrows_d16(N);
+        case 32: return mfma_dqr_qrows_d32(N);
+        case 64: return mfma_dqr_qrows_d64(N);
     }
     return 0;
 }

@@ -8,7 +8,8 @@
 // is how the per-row operands arrive.  There, every S row starts with loads whose latency
 // nothing hides (a few microseconds, several times the arithmetic of the row).  Here
 //   * the workgroup has 8 waves and a slab of 64 query rows: wave w works on query tile
-//     w / 4 and, of every block of keys, on the 32-key tiles (w % 4), (w % 4) + 4, ...;
+//     w / 4 and, of every block of keys, on the 32-key tiles (w % 4), (w % 4) + 4, ... (for
+//     rows of more than one key block: 32 query rows, wave w on the key tiles w, w + 8, ...);
 //   * K, V, the mask columns, and the slab's Q, dO and O rows of S row s+1 are requested
 //     (16 bytes per lane and load, 6 loads per wave at D = 32) before row s is computed out
 //     of one LDS buffer, and written to the other buffer when that arithmetic is done; rows
@@ -31,14 +32,17 @@ namespace evo {
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-template <int D>
+// QT: 32-row query tiles per workgroup (2, or 1 for rows of several key blocks: half the
+// resident bias tiles and dBias accumulators per wave).
+template <int D, int QT>
 struct RingGeo {
     static constexpr int C = D / 8;                          // 16-byte chunks per row
     static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
     static constexpr int BKV = D <= 32 ? 256 : 128;          // keys per stage
     static constexpr int TPB = BKV / 32;                     // key tiles per stage
-    static constexpr int TPW = TPB / 4;                      // key tiles per stage and wave
-    static constexpr int QR = 64;                            // query rows per workgroup
+    static constexpr int KQ = 8 / QT;                        // waves per query tile, each with key tiles of its own
+    static constexpr int TPW = TPB / KQ;                     // key tiles per stage and wave
+    static constexpr int QR = 32 * QT;                       // query rows per workgroup
     static constexpr int DP = (D + 31) / 32 * 32;
     static constexpr int RP = DP + 4;                        // pitch of a partial dQ row (floats)
     static constexpr int K_BYTES = BKV * D * 2;
@@ -80,12 +84,13 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #define EVO_TR(slot) do {} while (0)
 #endif
 
-template <typename T, int D, bool HAS_BIAS, int NBLK>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT>
 __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
-    typedef RingGeo<D> R;
+    typedef RingGeo<D, QT> R;
+    static_assert(R::TPW >= 1 && R::Q_BYTES % 1024 == 0, "query slab too small for this head dim");
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
-    constexpr int C = R::C, BKV = R::BKV, TPB = R::TPB, TPW = R::TPW, RP = R::RP;
+    constexpr int C = R::C, BKV = R::BKV, TPB = R::TPB, TPW = R::TPW, RP = R::RP, KQ = R::KQ, QR = R::QR;
     constexpr int NSLOT = NBLK * TPW;   // key tiles per wave over a whole row
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v4 v4;
@@ -95,15 +100,15 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar, so that what depends on it branches
     const int li = lane & 31, g = lane >> 5;
-    const int qi = wave >> 2, kq = wave & 3;
-    const int NT = (p.N + 31) / 32, NQP = (NT + 1) / 2;
+    const int qi = wave / KQ, kq = wave % KQ;
+    const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
     const int np256 = (p.N + 255) / 256 * 256;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const int qp = lid % NQP;
     const unsigned bh = (lid / NQP) % (unsigned)(p.B * p.H);
     const int c = lid / NQP / (unsigned)(p.B * p.H);
     const int b = bh / p.H, h = bh % p.H;
-    const int qbase = qp * 64;
+    const int qbase = qp * QR;
     const int q0 = qbase + qi * 32;
     const bool qact = q0 < p.N;             // wave-uniform; an odd tile count leaves one pair half empty
     const int qt = min(q0 >> 5, NT - 1);
@@ -119,7 +124,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
 
     // key tile of slot j of this wave
-    auto slot_tile = [&](int j) { return (j / TPW) * TPB + (j % TPW) * 4 + kq; };
+    auto slot_tile = [&](int j) { return (j / TPW) * TPB + (j % TPW) * KQ + kq; };
 
     f32x16 bres[HAS_BIAS ? NSLOT : 1];
     if (HAS_BIAS) {
@@ -224,35 +229,37 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
             }
         }
-        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total)
+        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR)
             *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
     };
     auto stash = [&](int t) { stash_part(t, 0, IPW); };
 
-    // The four partial dQ^T tiles of a query tile (one per wave, fp32, in the buffer of the
+    // The partial dQ^T tiles of a query tile (one per wave that works on it, fp32, in the buffer of the
     // stage they came from) summed, scaled and stored as row `base` of dQ.
     auto sum_store = [&](const float *red, int64_t base) {
         T *dQ = (T *)p.dq + base;
-        for (int it = tid; it < 64 * (D / 4); it += 512) {
+        for (int it = tid; it < QR * (D / 4); it += 512) {
             const int q = it / (D / 4), d4 = (it % (D / 4)) * 4;
-            const int w0 = (q >> 5) * 4, ql = q & 31;
+            const int w0 = (q >> 5) * KQ, ql = q & 31;
             f32x4 sum = *reinterpret_cast<const f32x4 *>(&red[(w0 * 32 + ql) * RP + d4]);
 #pragma unroll
-            for (int w = 1; w < 4; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
+            for (int w = 1; w < KQ; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
             if (qbase + q < p.N)
                 store4<T>(dQ + (int64_t)(qbase + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
                           sum[3] * p.scale);
         }
     };
-    // With one key block per row the sum of a row's partials waits until the next row's stage
-    // barrier has been passed (two barriers per row instead of three): nobody writes where the
-    // partials lie before the barrier that follows the next row's tiles.
-    constexpr bool DEFER = NBLK == 1;
+    // The sum of a row's partials waits until the next row's first stage barrier has been
+    // passed: nobody writes where the partials lie before another barrier has followed, which
+    // with several key blocks per row is the next stage barrier and with one is a barrier of
+    // its own (XBAR) between the row's tiles and the write of its partials.
+    static_assert(NBLK == 1 || R::OWN_RED, "rows of several key blocks keep the partials out of the stage buffers");
+    constexpr bool XBAR = NBLK == 1;
     // With the partials out of the stage buffers, the buffer of the next stage is free from
     // the stage barrier on: every wave asks for half of its pieces at the top of the row and
     // writes them to LDS between its two tiles, while other waves compute; the other half it
     // asks for after the row's prologue and writes after the tiles.
-    constexpr bool MID = DEFER && R::OWN_RED && TPW >= 2;
+    constexpr bool MID = NBLK == 1 && R::OWN_RED && TPW >= 2;
     auto red_of = [&](int stage) { return (float *)(lds + (R::OWN_RED ? 2 * R::BUF_BYTES : (stage & 1) * R::BUF_BYTES)); };
 
     fetch(0);
@@ -293,8 +300,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             else if (early) fetch(t + 1);
             EVO_TR(3);
             buf = lds + (t & 1) * R::BUF_BYTES;
-            if (DEFER && s > s_begin)
-                sum_store(red_of(t - 1), pr.base - p.stride_s);
+            if (blk == 0 && s > s_begin) sum_store(red_of(t - 1), pr.base - p.stride_s);
 
             if (blk == 0) {
                 // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
@@ -342,7 +348,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
-                    const int tb = jj * 4 + kq;          // tile inside the stage
+                    const int tb = jj * KQ + kq;         // tile inside the stage
                     const int kt = blk * TPB + tb;
                     if (MID && jj == TPW - 1) stash_part(t + 1, 0, SPLIT);
                     if (qact && kt < NT) {  // wave-uniform
@@ -414,13 +420,13 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             }
             // into the other buffer, free since the barrier above
             if (MID) stash_part(t + 1, SPLIT, IPW);
-            else if (!DEFER) stash(t + 1);
+            else if (R::OWN_RED) stash(t + 1);
         }
 
         // Partial dQ^T of this wave: lane = query li, register r = dim dt*32 + crow(r, g).  The
-        // four waves of a query tile meet in the buffer of the stage just consumed.
+        // waves of a query tile meet in LDS.
         EVO_TR(5);
-        lds_barrier();
+        if (XBAR) lds_barrier();
         EVO_TR(6);
         float *red = red_of(t - 1);
 #pragma unroll
@@ -433,20 +439,13 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 *reinterpret_cast<f32x4 *>(&red[(wave * 32 + li) * RP + dt * 32 + 8 * rr + 4 * g]) = v;
             }
         EVO_TR(7);
-        if (DEFER) {
-            // the other buffer held the last row's partials; everyone has summed them by now
-            if (!MID) stash(t);
-            EVO_TR(8);
-        } else {
-            lds_barrier();
-            EVO_TR(8);
-            sum_store(red, pr.base);
-        }
+        // where the partials share the stage buffers, the other buffer held the last row's;
+        // everyone has summed them by now
+        if (!R::OWN_RED) stash(t);
+        EVO_TR(8);
         EVO_TR(9);
-        // the barrier at the top of the next stage keeps the next request for this buffer
-        // behind these reads
     }
-    if (DEFER && s_end > s_begin) {
+    if (s_end > s_begin) {
         lds_barrier();
         sum_store(red_of(t - 1), base0 + (int64_t)(s_end - 1 - s_begin) * p.stride_s);
     }
@@ -479,35 +478,48 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, bool HAS_BIAS, int NBLK>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT>
 static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    typedef RingGeo<D> R;
+    typedef RingGeo<D, QT> R;
     static bool attr_set = false;
-    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK>;
+    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT>;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES) != hipSuccess)
             return EVO_EHIP;
         attr_set = true;
     }
-    const int NT = (p.N + 31) / 32, NQP = (NT + 1) / 2;
+    const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
     const unsigned grid = (unsigned)NQP * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
     kern<<<grid, 512, R::LDS_BYTES, st>>>(p, e);
     return hip_rc();
 }
 
-// Key blocks per row the kernel is built for: with more, the resident bias tiles and dBias
-// accumulators (16 registers each per key tile and wave) no longer fit 256 registers, and the
-// spilled form measured slower than the one-workgroup-per-problem kernel (N = 384, D = 32).
+// The forms the kernel is built in.  Per key tile of a row a wave keeps 16 registers of bias
+// and 16 of dBias sums, so rows of one key block run with two query tiles per workgroup (two
+// key tiles per wave); longer rows run with one query tile per workgroup (one key tile per
+// wave and block, up to three blocks: with more the spilled form is slower than the
+// one-workgroup-per-problem kernel), head dim 8 up to two blocks with two query tiles.
 template <int D>
-constexpr int dqr_max_blocks() { return D == 8 ? 2 : 1; }
+constexpr int dqr_key_blocks(int n) { return (n + RingGeo<D, 2>::BKV - 1) / RingGeo<D, 2>::BKV; }
+template <int D>
+constexpr int dqr_query_tiles(int n) {
+    const int nblk = dqr_key_blocks<D>(n);
+    if (nblk == 1) return 2;
+    if (D == 8) return nblk == 2 ? 2 : 0;
+    if (D == 16 || D == 32) return nblk <= 3 ? 1 : 0;
+    return 0;
+}
 
 template <typename T, int D, bool HAS_BIAS>
 static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    typedef RingGeo<D> R;
-    const int nblk = (p.N + R::BKV - 1) / R::BKV;
-    if (nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1>(p, e, st);
-    if constexpr (dqr_max_blocks<D>() >= 2) {
-        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2>(p, e, st);
+    const int nblk = dqr_key_blocks<D>(p.N);
+    if (nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2>(p, e, st);
+    if constexpr (D == 8) {
+        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 2>(p, e, st);
+    }
+    if constexpr (D == 16 || D == 32) {
+        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 1>(p, e, st);
+        if (nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3, 1>(p, e, st);
     }
     return EVO_EUNSUPPORTED;
 }
@@ -517,8 +529,9 @@ static int dqr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.bias_dtype == EVO_NONE ? dqr_blocks<T, D, false>(p, e, st) : dqr_blocks<T, D, true>(p, e, st);
 }
 
-// Largest N the double-buffered dQ kernel takes for this head dim.
-int EVO_CAT(mfma_dqr_max_n_d, EVO_D)() { return dqr_max_blocks<EVO_D>() * RingGeo<EVO_D>::BKV; }
+// Query rows one workgroup of the double-buffered dQ kernel takes at this N (64 or 32); 0
+// where the kernel is not built for such rows.
+int EVO_CAT(mfma_dqr_qrows_d, EVO_D)(int n) { return 32 * dqr_query_tiles<EVO_D>(n); }
 
 int EVO_CAT(launch_mfma_dqr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.dtype == EVO_BF16 ? dqr_bias<bf16_t, EVO_D>(p, e, st) : dqr_bias<f16_t, EVO_D>(p, e, st);
