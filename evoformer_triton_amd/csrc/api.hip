@@ -92,7 +92,7 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
 }
 
 struct PrepLayout {
-    size_t bq, bk, m2, m2a, dead, total;
+    size_t bq, bk, bt, m2, m2a, dead, total;
     int bias_batches;
 };
 
@@ -105,6 +105,10 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
     size_t off = 0;
     w.bq = off; off += align_up(tiles);
     w.bk = off; off += align_up(tiles);
+    // transposed 16-bit copy for the kernels that keep bias columns resident
+    const bool bt_ok = p.bias && p.bias_dtype == p.dtype && p.N % 8 == 0;
+    w.bt = bt_ok ? off : (size_t)-1;
+    if (bt_ok) off += align_up((size_t)w.bias_batches * p.H * p.N * p.N * 2);
     w.m2 = off; off += align_up((size_t)p.B * p.S * NT * 32 * 8);
     w.m2a = off; off += align_up((size_t)p.B * p.S * ((p.N + 255) / 256 * 256) * 16);
     w.dead = off; off += align_up((size_t)p.B * p.S * 4);
@@ -118,6 +122,7 @@ static void fill_prep(const EvoAttnParams &p, Extra &e) {
     e.bias_batches = w.bias_batches;
     e.bq = (float *)(base + w.bq);
     e.bk = (float *)(base + w.bk);
+    e.bt = w.bt == (size_t)-1 ? nullptr : (void *)(base + w.bt);
     e.m2 = (uint2 *)(base + w.m2);
     e.m2a = (uint4 *)(base + w.m2a);
     e.dead = (int *)(base + w.dead);
@@ -221,10 +226,19 @@ static bool fwd_ring_ok(const EvoAttnParams &p) {
     return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
 }
 
+// The dK/dV kernel that walks over a chunk of S rows keeps 16-bit bias columns resident: it
+// takes a bias in the dtype of q (or none) and rows whose length is a multiple of 8.  Bit
+// 0x200 of flags (not part of the public interface) selects the other kernel, for comparison.
+static bool kv_ring_ok(const EvoAttnParams &p) {
+    if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x200)) || p.N <= 128 || p.N > mfma_kvr_max_n(p.D) || p.N % 8) return false;
+    return !p.bias || p.bias_dtype == p.dtype;
+}
+
 const char *evoattn_kernels(const EvoAttnParams *p, int pass) {
     if (!p) return "invalid";
     if (!mfma_ok(*p, pass)) return "generic";
     if (pass == EVO_PASS_FWD) return fwd_ring_ok(*p) ? "mfma_fwd_ring" : "mfma_fwd";
+    if (kv_ring_ok(*p)) return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv_ring" : "mfma_dq,mfma_dkdv_ring";
     return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv" : "mfma_dq,mfma_dkdv";
 }
 
@@ -264,10 +278,11 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
     const bool ring = dq_ring_ok(*p);
     if (p->flags & EVO_FLAG_ONLY_DQ) return ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st);
-    if (p->flags & EVO_FLAG_ONLY_DKDV) return launch_mfma_dkdv(*p, e, st);
+    const bool kvring = kv_ring_ok(*p);
+    if (p->flags & EVO_FLAG_ONLY_DKDV) return kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads
     if ((rc = ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st))) return rc;
-    if ((rc = launch_mfma_dkdv(*p, e, st))) return rc;
+    if ((rc = kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st))) return rc;
     if (p->dbias && (rc = launch_dbias_reduce(*p, e, st))) return rc;
     if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;
     return EVO_OK;

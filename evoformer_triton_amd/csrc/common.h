@@ -46,6 +46,8 @@ struct Extra {
     uint2 *m2;         // additive mask * log2(e), shifted, clamped, as (hi, mid, lo, 0) of T  [B][S][NT*32]
     uint4 *m2a;        // the same mask rows as ready-made 16-byte operand chunks (hi, mid, lo, 1, 1, 1, 0, 0),
                        // padded with the floor to a multiple of 256 keys                        [B][S][NP256]
+    void *bt;          // the bias transposed (key-major), in the dtype of q; null unless the bias has
+                       // that dtype and N is a multiple of 8                                    [Bb][H][N][N]
     int *dead;         // [B][S] 1 where every key of the row is masked out
     int64_t zero_tile; // offset (floats) of an all-zero tile inside bq and bk
     long long *trace;  // trace builds only: 16 timestamps per wave

@@ -11,6 +11,8 @@ namespace evo {
     int launch_mfma_dq_d##D(const EvoAttnParams &, const Extra &, hipStream_t);              \
     int launch_mfma_dqr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
     int mfma_dqr_qrows_d##D(int);                                                            \
+    int launch_mfma_kvr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
+    int mfma_kvr_max_n_d##D();                                                               \
     int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
 EVO_DECL(16)
@@ -32,6 +34,7 @@ EVO_ROUTE(fwd)
 EVO_ROUTE(fwdr)
 EVO_ROUTE(dq)
 EVO_ROUTE(dqr)
+EVO_ROUTE(kvr)
 EVO_ROUTE(dkdv)
 #undef EVO_ROUTE
 
@@ -41,6 +44,16 @@ int mfma_fwdr_max_n(int D) {
         case 16: return mfma_fwdr_max_n_d16();
         case 32: return mfma_fwdr_max_n_d32();
         case 64: return mfma_fwdr_max_n_d64();
+    }
+    return 0;
+}
+
+int mfma_kvr_max_n(int D) {
+    switch (D) {
+        case 8: return mfma_kvr_max_n_d8();
+        case 16: return mfma_kvr_max_n_d16();
+        case 32: return mfma_kvr_max_n_d32();
+        case 64: return mfma_kvr_max_n_d64();
     }
     return 0;
 }

@@ -59,6 +59,20 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
         const int64_t o = ((int64_t)t * 64 + lane) * 16 + 4 * rr;
         *reinterpret_cast<f32x4 *>(e.bq + o) = vq;
         *reinterpret_cast<f32x4 *>(e.bk + o) = vk;
+        if (e.bt) {
+            // the same four entries of column `key` as given (the dtypes agree, so exact),
+            // key-major: N is a multiple of 8 here, so the four are inside the matrix or not
+            const int q = qt * 32 + 8 * rr + 4 * g, key = kt * 32 + li;
+            if (q < p.N && key < p.N) {
+                const int64_t src = base + (int64_t)q * p.bias_stride_row + key;
+                const int64_t dst = (((int64_t)bb * p.H + h) * p.N + key) * p.N + q;
+                unsigned short w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w[i] = ((const unsigned short *)p.bias)[src + (int64_t)i * p.bias_stride_row];
+                *reinterpret_cast<uint2 *>((unsigned short *)e.bt + dst) =
+                    make_uint2(w[0] | ((unsigned)w[1] << 16), w[2] | ((unsigned)w[3] << 16));
+            }
+        }
         return;
     }
     const unsigned row = blockIdx.x - n_bias_blocks;  // (b, s)
