@@ -227,6 +227,22 @@ __device__ __forceinline__ float dot8<f16_t>(f16x8 a, f16x8 b, float acc) {
     return acc;
 }
 
+// The two 16-bit values of a packed pair as fp32.
+template <typename T>
+__device__ __forceinline__ void unpack2(unsigned w, float &lo, float &hi);
+template <>
+__device__ __forceinline__ void unpack2<bf16_t>(unsigned w, float &lo, float &hi) {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ void unpack2<f16_t>(unsigned w, float &lo, float &hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 v = __builtin_bit_cast(h2, w);
+    lo = (float)v[0];
+    hi = (float)v[1];
+}
+
 // (hi, mid, lo, 0) of split3 packed into 8 bytes.
 template <typename T>
 __device__ __forceinline__ uint2 pack_split3(float m) {

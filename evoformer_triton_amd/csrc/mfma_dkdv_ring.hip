@@ -49,22 +49,6 @@ struct KvRingGeo {
     static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
 };
 
-// The two 16-bit values of a packed pair as fp32.
-template <typename T>
-__device__ __forceinline__ void unpack2(unsigned w, float &lo, float &hi);
-template <>
-__device__ __forceinline__ void unpack2<bf16_t>(unsigned w, float &lo, float &hi) {
-    lo = __uint_as_float(w << 16);
-    hi = __uint_as_float(w & 0xffff0000u);
-}
-template <>
-__device__ __forceinline__ void unpack2<f16_t>(unsigned w, float &lo, float &hi) {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const h2 v = __builtin_bit_cast(h2, w);
-    lo = (float)v[0];
-    hi = (float)v[1];
-}
-
 __device__ __forceinline__ void lds_barrier_kv() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 template <typename T, int D, bool HAS_BIAS>
