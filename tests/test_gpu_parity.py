@@ -220,6 +220,21 @@ def test_small_cases_bf16(E, case):
     assert_close(got, ref, BF16_TOL, ["O", "dQ", "dK", "dV", "dBias"] + (["dMask"] if fmask else []), what=str(case))
 
 
+@pytest.mark.parametrize("case", [(1, 6, 256, 2, 32, "add", "q"), (1, 5, 200, 2, 32, "soft", "q"),
+                                  (2, 4, 144, 2, 32, "bool", None), (1, 3, 384, 2, 32, "add", "q")],
+                         ids=lambda c: "-".join(map(str, c)))
+def test_small_cases_fp16(E, case):
+    """The fp16 instantiations of the chunk-of-rows kernels (N = 129..256: forward, dQ, dK/dV with
+    the bias columns unpacked from fp16 pairs; N = 384: dQ with two key blocks per row) against the
+    CPU oracle in fp32 on the same fp16 inputs."""
+    B, S, N, H, D, mask, bias_dt = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, torch.float16, seed=5)
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
+    fmask = m is not None and m.dtype != torch.bool
+    got = run_hip(E, Q, K, V, m, bias, dO, mask_grad=fmask)
+    assert_close(got, ref, 4e-3, ["O", "dQ", "dK", "dV", "dBias"] + (["dMask"] if fmask else []), what=str(case))
+
+
 @pytest.mark.parametrize("shape,mask", [((1, 37, 256, 2, 32), "add"), ((1, 5, 200, 3, 16), "bool"),
                                         ((2, 3, 130, 2, 8), "soft"), ((1, 4, 384, 2, 32), "add"),
                                         ((1, 3, 480, 1, 64), "add")])
