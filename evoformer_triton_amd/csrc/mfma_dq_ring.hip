@@ -53,8 +53,8 @@ struct RingGeo {
     static constexpr int OFF_Q = OFF_A + A_BYTES;
     static constexpr int OFF_G = OFF_Q + Q_BYTES;
     static constexpr int OFF_O = OFF_G + Q_BYTES;
-    static constexpr int OFF_L = OFF_O + Q_BYTES;                   // log-sum-exp of the QR query rows, fp32
-    static constexpr int STAGE_BYTES = OFF_L + QR * 4;
+    static constexpr int OFF_L = OFF_O + Q_BYTES;                   // -log2-sum-exp of the QR query rows as (hi, mid, lo, 0)
+    static constexpr int STAGE_BYTES = OFF_L + QR * 8;
     static constexpr int RED_BYTES = 8 * 32 * RP * 4;
     static constexpr int STAGE_1K = (STAGE_BYTES + 1023) / 1024 * 1024;
     // The partial dQ tiles get LDS of their own where 160 KB allow it; otherwise they lie in the
@@ -142,7 +142,8 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     }
 
     const int s_begin = c * e.chunk, s_end = min(p.S, s_begin + e.chunk);
-    const int T_total = (s_end - s_begin) * NBLK;
+    const int nrows = s_end - s_begin;
+    const int T_total = nrows * NBLK;
 
     // ---- stage t = (row s_begin + t / NBLK, key block t % NBLK) lives in buffer t & 1.  It is a
     // list of 1 KB pieces (64 lanes x 16 bytes); piece n belongs to wave n % 8.  Lane i of
@@ -216,21 +217,31 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     };
     auto fetch = [&](int t) { fetch_part(t, 0, IPW); };
     constexpr int SPLIT = IPW / 2;   // pieces asked for at the top of a row; the rest after its prologue
+    // What every wave of a query tile would otherwise redo in its prologue is done once, by
+    // the wave that writes the piece: Q goes to LDS scaled by scale*log2(e) (where the scaled
+    // Q is rounded once; with the rounding residue carried along it goes as given), zeroed
+    // for a row with every key masked, and the log-sum-exp as its three operand columns.
+    constexpr bool PRESCALE = !G::RESID;
+    bool stage_dead = PRESCALE && uniform_load(e.dead + b * p.S + s_begin) != 0;
     auto stash_part = [&](int t, int i0, int i1) {
         const int blk = t % NBLK;
         const int ninst = t >= T_total ? 0 : blk == 0 ? R::I_ALL : R::I_KVA;
         unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+        const float cq = stage_dead ? 0.0f : cs;   // (the flag of the row this stage belongs to)
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             if (i < i0 || i >= i1) continue;
             const int n = wave + 8 * i;
             if (n < ninst) {
                 const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
-                *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
+                if (PRESCALE && n >= R::I_KVA && n < R::I_KVA + R::I_Q)
+                    *reinterpret_cast<v8 *>(buf + dst + lane * 16) = scaled8<T>(__builtin_bit_cast(v8, stg[i]), cq);
+                else
+                    *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
             }
         }
         if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR)
-            *reinterpret_cast<float *>(buf + R::OFF_L + lane * 4) = lse_stg;
+            *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-lse_stg * kLog2e);
     };
     auto stash = [&](int t) { stash_part(t, 0, IPW); };
 
@@ -276,6 +287,8 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         pr.row0 = (int64_t)pid * p.N;
         const bool dead = uniform_load(e.dead + b * p.S + s) != 0;
         const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
+        // for the stage with query rows that is written during this row: the next row's
+        stage_dead = PRESCALE && uniform_load(e.dead + b * p.S + min(s + 1, s_end - 1)) != 0;
 
         v8 qf[KS], gf[KS], qlo[KSD];
         f32x16 dqacc[DT];
@@ -304,7 +317,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
             if (blk == 0) {
                 // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
-                const float lse2 = *reinterpret_cast<const float *>(buf + R::OFF_L + (qi * 32 + li) * 4) * kLog2e;
+                const uint2 nlse3 = *reinterpret_cast<const uint2 *>(buf + R::OFF_L + (qi * 32 + li) * 8);
                 float dpart = 0.0f;
 #pragma unroll
                 for (int ks = 0; ks < KSD; ++ks) qlo[ks] = zero8<T>();
@@ -318,7 +331,8 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         const v8 qraw = *reinterpret_cast<const v8 *>(buf + R::OFF_Q + o);
                         gf[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_G + o);
                         const v8 oraw = *reinterpret_cast<const v8 *>(buf + R::OFF_O + o);
-                        if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
+                        if (PRESCALE) qf[ks] = qraw;   // scaled (and zeroed for a dead row) when it was staged
+                        else if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
                         dpart = dot8<T>(gf[ks], oraw, dpart);
                     }
                 }
@@ -332,7 +346,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     if (ks * 16 + g * 8 == AUGC) {
-                        qf[ks] = aug8<T>(one3, pack_split3<T>(-lse2));   // ones x mask, -lse x ones
+                        qf[ks] = aug8<T>(one3, nlse3);                   // ones x mask, -lse x ones
                         gf[ks] = aug8<T>(pack_split3<T>(-dl), zero3);    // -delta x ones
                     }
                 }
