@@ -231,6 +231,7 @@ static bool fwd_ring_ok(const EvoAttnParams &p) {
 // 0x200 of flags (not part of the public interface) selects the other kernel, for comparison.
 static bool kv_ring_ok(const EvoAttnParams &p) {
     if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x200)) || p.N <= 128 || p.N > mfma_kvr_max_n(p.D) || p.N % 8) return false;
+    if (!aligned(p.lse, 16)) return false;   // LSE rows are read four values at a time
     return !p.bias || p.bias_dtype == p.dtype;
 }
 
