@@ -188,6 +188,8 @@ SMALL = [
     (1, 5, 252, 2, 32, "bool", "q", "reference"),      # bias rows not 16-byte aligned: fp32 tiles
     (1, 5, 256, 2, 16, "soft", torch.float32, "reference"),
     (2, 3, 136, 2, 8, "add", "q", "reference"),
+    (1, 5, 200, 2, 32, "soft", "q", "reference"),      # dMask partials from the chunk-of-rows dK/dV
+    (2, 4, 168, 2, 32, "bool", None, "ds4sci"),        # the same kernel without bias, per-head strides
 ]
 
 
