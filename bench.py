@@ -51,10 +51,81 @@ def parse():
                          "takes some tenths of a second of load to reach its steady clocks, and a handful of "
                          "400-microsecond warm-up steps ends before that (measured: 8 % slower steps)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--reference-sweep", action="store_true",
+                    help="instead of the step benchmark: the reference's own speed benchmark (speed_benchmark.py:37-115: "
+                         "B=4, H=32, D=64, N_seq=1, bool mask, fp32 pair bias, modes fwd / bwd / full, timed like "
+                         "triton.testing.do_bench with the caches flushed before every repetition) on this build; "
+                         "prints one JSON line with TFLOP/s per N beside the numbers the reference publishes")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy three times: under rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
     return ap.parse_args()
+
+
+# fwd / bwd / fwd+bwd TFLOP/s the reference publishes for its Triton kernels (speed_benchmark.py:129-173; hardware
+# not stated, sm_80-class), N_CTX -> value
+PUBLISHED_TRITON = {
+    "fwd": {256: 34.14, 384: 42.74, 512: 50.84, 768: 59.10, 1024: 63.77, 2048: 73.07},
+    "bwd": {256: 10.71, 384: 11.67, 512: 12.26, 768: 12.68, 2048: 13.38},
+    "full": {256: 13.15, 384: 14.57, 512: 15.52, 768: 16.25, 2048: 17.42},
+}
+
+
+def reference_sweep():
+    """speed_benchmark.py:56-115 against this build: same shapes, dtypes, input distributions, FLOP
+    formula and timing scheme (warm-up, then repetitions each preceded by a write over a buffer larger
+    than the last-level cache, one event pair per repetition, mean)."""
+    import torch
+    from evoformer_triton_amd import EvoformerAttention
+    dev = torch.device("cuda:0")
+    BATCH, H, D, S = 4, 32, 64, 1
+    flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+
+    def do_bench(fn, warmup_ms=25.0, rep_ms=100.0):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            flush.zero_()
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        est = a.elapsed_time(b) / 5
+        for _ in range(max(1, int(warmup_ms / est))):
+            fn()
+        n = max(1, int(rep_ms / est))
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for s0, s1 in ev:
+            flush.zero_()
+            s0.record()
+            fn()
+            s1.record()
+        torch.cuda.synchronize()
+        return sum(s0.elapsed_time(s1) for s0, s1 in ev) / n
+
+    out = {}
+    for N in (256, 384, 512, 768, 1024, 2048):
+        q, k, v = (torch.randn((BATCH, S, N, H, D), dtype=torch.bfloat16, device=dev, requires_grad=True) for _ in range(3))
+        mask = torch.randint(0, 2, (BATCH, S, 1, 1, N), dtype=torch.bool, device=dev)
+        bias = torch.randn((BATCH, 1, H, N, N), dtype=torch.float32, device=dev)
+        fwd = lambda: EvoformerAttention.apply(q, k, v, mask, bias)
+        o = fwd()
+        do = torch.randn_like(o)
+        bwd = lambda: o.backward(do, retain_graph=True)
+
+        def full():
+            o2 = EvoformerAttention.apply(q, k, v, mask, bias)
+            o2.backward(torch.randn_like(o2), retain_graph=True)
+
+        mm = 2.0 * BATCH * H * N * N * D
+        row = {}
+        for mode, fn, mult in (("fwd", fwd, 2.0), ("bwd", bwd, 5.0), ("full", full, 7.0)):
+            ms = do_bench(fn)
+            row[mode] = {"ms": ms, "tflops": mult * mm * 1e-12 / (ms * 1e-3), "published_triton_tflops": PUBLISHED_TRITON[mode].get(N)}
+        out[str(N)] = row
+        q.grad = k.grad = v.grad = None
+    print(json.dumps({"reference_sweep": {"shape": "B=4 N_seq=1 H=32 D=64 bf16, bool mask, fp32 bias", "by_n": out}}))
 
 
 def cpu_baseline(cfg, shape, budget_s=15.0):
@@ -87,6 +158,8 @@ def main():
         print(f"bench.py: this build runs on one GPU; --gpus {args.gpus} is not supported "
               "(the path would shard over S with one dBias all-reduce)", file=sys.stderr)
         sys.exit(2)
+    if args.reference_sweep:
+        return reference_sweep()
     import torch
     from oracle import eager
     import evoformer_triton_amd.evoformer as E

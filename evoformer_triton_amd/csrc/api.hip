@@ -59,9 +59,22 @@ static int bias_vec_ok(const EvoAttnParams &p) {
     return aligned(p.bias, a) && p.bias_stride_b % 4 == 0 && p.bias_stride_h % 4 == 0 && p.bias_stride_row % 4 == 0;
 }
 
+// The prepared bias tiles (two fp32 copies in accumulator order) cost 12 bytes of memory traffic
+// per bias entry before any kernel has used one; each kernel then reads 4 bytes per entry and S
+// row.  With very few S rows per (batch, head) - the reference's own speed benchmark has one -
+// the one-workgroup-per-problem kernels read the caller's tensor instead, which needs rows that
+// allow 16-byte (fp32) or 8-byte loads.  Bit 0x800 of flags (not part of the public interface)
+// keeps the tiles, for comparison.
+static bool bias_direct(const EvoAttnParams &p) {
+    if (!p.bias || p.S > 4 || (p.flags & 0x800) || p.N % 4) return false;
+    if (p.bias_dtype != EVO_F32 && p.bias_dtype != p.dtype) return false;
+    if ((int64_t)p.N * p.bias_stride_row >= ((int64_t)1 << 31)) return false;   // 32-bit offsets inside one (b, h) matrix
+    return bias_vec_ok(p) != 0;
+}
+
 // The dQ kernel that double-buffers its operands in LDS takes rows of limited length.
 static bool dq_ring_ok(const EvoAttnParams &p) {
-    return !(p.flags & EVO_FLAG_PER_PROBLEM) && mfma_dqr_qrows(p.D, p.N) > 0;
+    return !(p.flags & EVO_FLAG_PER_PROBLEM) && !bias_direct(p) && mfma_dqr_qrows(p.D, p.N) > 0;
 }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
@@ -101,12 +114,12 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
     const size_t NT = (size_t)(p.N + 31) / 32;
     w.bias_batches = (p.bias && p.bias_stride_b == 0) ? 1 : p.B;
     // one extra all-zero tile at the end of each copy
-    const size_t tiles = p.bias ? ((size_t)w.bias_batches * p.H * NT * NT + 1) * 1024 * 4 : 0;
+    const size_t tiles = p.bias && !bias_direct(p) ? ((size_t)w.bias_batches * p.H * NT * NT + 1) * 1024 * 4 : 0;
     size_t off = 0;
     w.bq = off; off += align_up(tiles);
     w.bk = off; off += align_up(tiles);
     // transposed 16-bit copy for the kernels that keep bias columns resident
-    const bool bt_ok = p.bias && p.bias_dtype == p.dtype && p.N % 8 == 0;
+    const bool bt_ok = p.bias && !bias_direct(p) && p.bias_dtype == p.dtype && p.N % 8 == 0;
     w.bt = bt_ok ? off : (size_t)-1;
     if (bt_ok) off += align_up((size_t)w.bias_batches * p.H * p.N * p.N * 2);
     w.m2 = off; off += align_up((size_t)p.B * p.S * NT * 32 * 8);
@@ -120,6 +133,7 @@ static void fill_prep(const EvoAttnParams &p, Extra &e) {
     const PrepLayout w = prep_layout(p);
     char *base = (char *)p.prep;
     e.bias_batches = w.bias_batches;
+    e.bias_direct = bias_direct(p) ? 1 : 0;
     e.bq = (float *)(base + w.bq);
     e.bk = (float *)(base + w.bk);
     e.bt = w.bt == (size_t)-1 ? nullptr : (void *)(base + w.bt);
@@ -223,7 +237,7 @@ const char *evoattn_path(const EvoAttnParams *p, int pass) {
 
 // rows of 129..256 keys: a workgroup per chunk of S rows with the head's bias resident
 static bool fwd_ring_ok(const EvoAttnParams &p) {
-    return !(p.flags & EVO_FLAG_PER_PROBLEM) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
+    return !(p.flags & EVO_FLAG_PER_PROBLEM) && !bias_direct(p) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
 }
 
 // The dK/dV kernel that walks over a chunk of S rows keeps 16-bit bias columns resident: it
@@ -231,7 +245,7 @@ static bool fwd_ring_ok(const EvoAttnParams &p) {
 // 0x200 of flags (not part of the public interface) selects the other kernel, for comparison.
 static bool kv_ring_ok(const EvoAttnParams &p) {
     if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x200)) || p.N <= 128 || p.N > mfma_kvr_max_n(p.D) || p.N % 8) return false;
-    if (!aligned(p.lse, 16)) return false;   // LSE rows are read four values at a time
+    if (!aligned(p.lse, 16) || bias_direct(p)) return false;   // LSE rows are read four values at a time
     return !p.bias || p.bias_dtype == p.dtype;
 }
 

@@ -36,6 +36,7 @@ struct Extra {
     int chunk;         // rows of S per chunk
     int vec_ok;        // bias rows may be read with 8/16-byte vector loads
     int bias_batches;  // 1 when one bias is shared by the whole batch, else B
+    int bias_direct;   // the one-workgroup-per-problem kernels read the bias from the caller's tensor, not from bq / bk
     float *delta;      // [B][H][S][N]
     float *shift;      // [B][S] per-row mask shift (plain kernels)
     float *dbias_part; // [n_chunks][B][H][N][N]
@@ -241,6 +242,44 @@ __device__ __forceinline__ void unpack2<f16_t>(unsigned w, float &lo, float &hi)
     const h2 v = __builtin_bit_cast(h2, w);
     lo = (float)v[0];
     hi = (float)v[1];
+}
+
+// A 32x32 bias tile in accumulator order, times `mul`, straight from the caller's tensor (for
+// problems whose bias is used too few times to pay for the prepared fp32 tiles): `row` points
+// at this lane's own bias row (lane = row of the matrix, the tile's 32 columns start at c0;
+// entries 4 rr .. 4 rr + 3 are the columns c0 + 8 rr + 4 g ..).  The row must allow 16-byte
+// (fp32) or 8-byte (16-bit) loads at multiples of four columns; groups past column n repeat
+// the last whole group (such keys carry the mask floor).  F32: the tensor is fp32, else T.
+template <typename T, bool F32>
+__device__ __forceinline__ void bias_tile_rows(const void *row, int c0, int n, int g, float mul, f32x16 &dst) {
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const int col = min(c0 + 8 * rr + 4 * g, n - 4);
+        if (F32) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>((const float *)row + col);
+            dst[4 * rr] = v[0] * mul; dst[4 * rr + 1] = v[1] * mul; dst[4 * rr + 2] = v[2] * mul; dst[4 * rr + 3] = v[3] * mul;
+        } else {
+            const uint2 w = *reinterpret_cast<const uint2 *>((const T *)row + col);
+            float f0, f1, f2, f3;
+            unpack2<T>(w.x, f0, f1);
+            unpack2<T>(w.y, f2, f3);
+            dst[4 * rr] = f0 * mul; dst[4 * rr + 1] = f1 * mul; dst[4 * rr + 2] = f2 * mul; dst[4 * rr + 3] = f3 * mul;
+        }
+    }
+}
+
+// The same with lane = column of the matrix: `mat` points at element [0][0] (shared by the
+// lanes), `col` is this lane's column, the tile's 32 rows start at r0, consecutive rows are
+// `stride` elements apart (32-bit element offsets: the matrix has fewer than 2^31 entries); entry r
+// is the row r0 + crow(r, g), rows past n - 1 repeat the last one.
+template <typename T, bool F32>
+__device__ __forceinline__ void bias_tile_cols(const void *mat, unsigned col, int r0, int n, unsigned stride, int g, float mul,
+                                               f32x16 &dst) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const unsigned o = (unsigned)min(r0 + crow(r, g), n - 1) * stride + col;
+        dst[r] = (F32 ? ((const float *)mat)[o] : (float)((const T *)mat)[o]) * mul;
+    }
 }
 
 // (hi, mid, lo, 0) of split3 packed into 8 bytes.

@@ -90,7 +90,21 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
     const int bb = e.bias_batches > 1 ? b : 0;
     const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
     const float *ztile = e.bq + e.zero_tile + lane * 16;
-    auto load_btile = [&](const float *src, f32x16 &dst) {
+    // or, for a bias that is used too few times to pay for the tiles, this lane's row of the
+    // caller's tensor
+    const bool bdirect = HAS_BIAS && e.bias_direct;
+    const bool bf32 = p.bias_dtype == EVO_F32;
+    const char *brow = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h +
+                                               (int64_t)qrow * p.bias_stride_row) * (bf32 ? 4 : 2);
+    // key tile kt of this wave's query rows, in log2 units (zero for a row with every key masked)
+    auto load_btile = [&](int kt, bool dead_row, f32x16 &dst) {
+        if (bdirect) {   // uniform
+            const float mul = dead_row ? 0.0f : kLog2e;
+            if (bf32) bias_tile_rows<T, true>(brow, kt * 32, p.N, g, mul, dst);
+            else bias_tile_rows<T, false>(brow, kt * 32, p.N, g, mul, dst);
+            return;
+        }
+        const float *src = dead_row ? ztile : btile0 + (int64_t)kt * 1024;
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
@@ -100,7 +114,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
     f32x16 bres[NRES];
     if (BIAS_RESIDENT) {
 #pragma unroll
-        for (int j = 0; j < NRES; ++j) load_btile(btile0 + (int64_t)min(wave + 4 * j, NT - 1) * 1024, bres[j]);
+        for (int j = 0; j < NRES; ++j) load_btile(min(wave + 4 * j, NT - 1), false, bres[j]);
     }
 
     const uint2 one3 = ones3<T>();
@@ -193,7 +207,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
                             for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
                         }
                     } else {
-                        load_btile(dead ? ztile : btile0 + (int64_t)kt * 1024, acc);
+                        load_btile(kt, dead, acc);
                     }
                 }
 #pragma unroll
@@ -381,8 +395,17 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnPar
     const float *btile = dead ? e.bk + e.zero_tile + lane * 16
                               : e.bk + (((int64_t)bb * p.H + pr.h) * NT * NT + ktc) * 1024 + lane * 16;
     const int64_t bstep = dead ? 0 : (int64_t)NT * 1024;  // next query tile, same key tile
+    // or, for a bias that is used too few times to pay for the tiles, this lane's column of
+    // the caller's tensor
+    const bool bdirect = HAS_BIAS && e.bias_direct;
+    const bool bf32 = p.bias_dtype == EVO_F32;
+    const char *bmat = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h) * (bf32 ? 4 : 2);
+    const float bmul = dead ? 0.0f : kLog2e;
     auto load_btile = [&](int qt, f32x16 &dst) {
-        if (HAS_BIAS) {
+        if (HAS_BIAS && bdirect) {   // uniform
+            if (bf32) bias_tile_cols<T, true>(bmat, keyc, min(qt, NT - 1) * 32, p.N, (unsigned)p.bias_stride_row, g, bmul, dst);
+            else bias_tile_cols<T, false>(bmat, keyc, min(qt, NT - 1) * 32, p.N, (unsigned)p.bias_stride_row, g, bmul, dst);
+        } else if (HAS_BIAS) {
             const float *src = btile + (int64_t)min(qt, NT - 1) * bstep;
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {

@@ -99,6 +99,13 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_fwd(EvoAttnPara
     const float *btile = dead ? e.bq + e.zero_tile + lane * 16
                               : e.bq + ((((int64_t)bb * p.H + pr.h) * NT + qt) * NT) * 1024 + lane * 16;
     const int64_t bstep = dead ? 0 : 1024;
+    // or, for a bias that is used too few times to pay for the tiles, this lane's row of the
+    // caller's tensor
+    const bool bdirect = HAS_BIAS && e.bias_direct;
+    const bool bf32 = p.bias_dtype == EVO_F32;
+    const char *brow = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h +
+                                               (int64_t)qrow * p.bias_stride_row) * (bf32 ? 4 : 2);
+    const float bmul = dead ? 0.0f : kLog2e;
 
     float m = -INFINITY, l = 0.0f;
     f32x16 oacc[DT];
@@ -110,7 +117,10 @@ __global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_fwd(EvoAttnPara
     // Bias tile kt into 16 registers; past the last tile the previous one is read again
     // (every key there carries the mask floor, so the values do not matter).
     auto load_btile = [&](int kt, f32x16 &dst) {
-        if (HAS_BIAS) {
+        if (HAS_BIAS && bdirect) {   // uniform
+            if (bf32) bias_tile_rows<T, true>(brow, min(kt, NT - 1) * 32, p.N, g, bmul, dst);
+            else bias_tile_rows<T, false>(brow, min(kt, NT - 1) * 32, p.N, g, bmul, dst);
+        } else if (HAS_BIAS) {
             const float *src = btile + (int64_t)min(kt, NT - 1) * bstep;
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {

@@ -110,7 +110,8 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
 
 int launch_prep(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned NT = (p.N + 31) / 32;
-    const unsigned nb = p.bias ? (unsigned)e.bias_batches * p.H * NT * NT + 1u : 0u;
+    // (no bias tiles where the kernels read the caller's tensor)
+    const unsigned nb = p.bias && !e.bias_direct ? (unsigned)e.bias_batches * p.H * NT * NT + 1u : 0u;
     const unsigned nm = (unsigned)(p.B * p.S);
     prep_kernel<<<nb + nm, 256, 0, st>>>(p, e, nb);
     hipError_t err = hipGetLastError();
