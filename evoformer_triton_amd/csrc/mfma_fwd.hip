@@ -272,7 +272,14 @@ static int fwd_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 template <typename T, int D>
 static int fwd_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const int rem = p.N % 256;
-    const bool wide = p.N >= 256 && (rem == 0 || rem > 128);
+    bool wide = p.N >= 256 && (rem == 0 || rem > 128);
+    // ... and unless there are too few problems for that: below four workgroups per CU (256
+    // CUs) the narrower form's twice as many workgroups fill the chip better (the reference's
+    // speed benchmark has 128 problems).  Bit 0x100 of flags (not part of the public
+    // interface) inverts the choice, for comparison.
+    const int64_t wgs = (int64_t)((p.N + 255) / 256) * p.B * p.H * p.S;
+    if (wgs < 1024) wide = false;
+    if (p.flags & 0x100) wide = !wide;
     return wide ? fwd_bias<T, D, 8>(p, e, st) : fwd_bias<T, D, 4>(p, e, st);
 }
 
