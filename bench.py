@@ -125,7 +125,30 @@ def reference_sweep():
             row[mode] = {"ms": ms, "tflops": mult * mm * 1e-12 / (ms * 1e-3), "published_triton_tflops": PUBLISHED_TRITON[mode].get(N)}
         out[str(N)] = row
         q.grad = k.grad = v.grad = None
-    print(json.dumps({"reference_sweep": {"shape": "B=4 N_seq=1 H=32 D=64 bf16, bool mask, fp32 bias", "by_n": out}}))
+    del q, k, v, mask, bias, o, do, fwd, bwd, full, flush
+    # memory_benchmark.py:11-22, 38-39: max memory allocated after one forward+backward, bf16 bias without
+    # requires_grad, the same four-by-one-by-N-by-32-by-64 inputs; published (:46-53) for Triton / DS4Sci / torch
+    published_gb = {128: (0.2502, 0.0236, 0.0686), 256: (0.2698, 0.0549, 0.1995), 384: (0.2972, 0.0941, 0.4085),
+                    512: (0.3324, 0.1411, 0.6956), 768: (0.6570, 0.2586, 1.5042), 1024: (1.1260, 0.4072, 2.6253),
+                    2048: (4.2520, 1.3145, 10.2346)}
+    mem = {}
+    for N, pub in published_gb.items():
+        torch.cuda.synchronize()
+        del_list = None
+        torch.cuda.empty_cache()
+        base = torch.cuda.memory_allocated()
+        torch.cuda.reset_peak_memory_stats()
+        q, k, v = (torch.randn((BATCH, S, N, H, D), dtype=torch.bfloat16, device=dev, requires_grad=True) for _ in range(3))
+        mask = torch.randint(0, 2, (BATCH, S, 1, 1, N), dtype=torch.bool, device=dev)
+        bias = torch.randn((BATCH, 1, H, N, N), dtype=torch.bfloat16, device=dev)
+        o = EvoformerAttention.apply(q, k, v, mask, bias)
+        o.backward(torch.randn_like(o), retain_graph=True)
+        torch.cuda.synchronize()
+        mem[str(N)] = {"max_allocated_gb": (torch.cuda.max_memory_allocated() - base) / 1e9,
+                       "published_gb_triton_ds4sci_torch": pub}
+        del q, k, v, mask, bias, o
+    print(json.dumps({"reference_sweep": {"shape": "B=4 N_seq=1 H=32 D=64 bf16, bool mask, fp32 bias", "by_n": out,
+                                          "peak_memory_bf16_bias": mem}}))
 
 
 def cpu_baseline(cfg, shape, budget_s=15.0):
