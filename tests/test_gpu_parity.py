@@ -259,6 +259,25 @@ def test_chunk_of_rows_kernels_match_per_problem_kernels(E, shape, mask):
         assert max_err(a[name], b[name]) <= tol, (name, max_err(a[name], b[name]))
 
 
+@pytest.mark.parametrize("shape,bias_dt", [((2, 3, 200, 2, 32), torch.float32), ((1, 1, 384, 3, 64), "q"),
+                                           ((1, 4, 96, 2, 16), "q"), ((2, 2, 520, 1, 8), torch.float32)])
+def test_bias_read_from_the_callers_tensor_matches_the_prepared_tiles(E, shape, bias_dt):
+    """With at most four S rows the kernels read the pair bias from the caller's tensor instead of
+    the prepared fp32 tiles (flag bit 0x800 keeps the tiles): the same fp32 product bias x log2(e)
+    enters the same MFMA, so the two forms agree to the last bit."""
+    B, S, N, H, D = shape
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, "bool", bias_dt, torch.bfloat16, seed=9)
+    from evoformer_triton_amd import _lib
+    try:
+        E.FLAGS = 0x800 | _lib.EVO_FLAG_PER_PROBLEM      # the same one-workgroup-per-problem kernels, fed from tiles
+        a = run_hip(E, Q, K, V, m, bias, dO)
+    finally:
+        E.FLAGS = 0
+    b = run_hip(E, Q, K, V, m, bias, dO)
+    for name in a:
+        assert torch.equal(a[name], b[name]), (name, max_err(a[name], b[name]))
+
+
 def test_c1_fp32_check_mode_against_cpu_eager(E):
     x = eager.make_inputs("C1")
     ref = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"])     # fp32, as specified
