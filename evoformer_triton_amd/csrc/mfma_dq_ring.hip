@@ -34,11 +34,13 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // QT: 32-row query tiles per workgroup (2, or 1 for rows of several key blocks: half the
 // resident bias tiles and dBias accumulators per wave).
-template <int D, int QT>
+// KB: keys per stage (256, or 128: for head dim 64, whose rows are long, and for rows of 257..384
+// keys, which three blocks of 128 cover without an empty half block).
+template <int D, int QT, int KB>
 struct RingGeo {
     static constexpr int C = D / 8;                          // 16-byte chunks per row
     static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
-    static constexpr int BKV = D <= 32 ? 256 : 128;          // keys per stage
+    static constexpr int BKV = KB;                           // keys per stage
     static constexpr int TPB = BKV / 32;                     // key tiles per stage
     static constexpr int KQ = 8 / QT;                        // waves per query tile, each with key tiles of its own
     static constexpr int TPW = TPB / KQ;                     // key tiles per stage and wave
@@ -84,10 +86,10 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #define EVO_TR(slot) do {} while (0)
 #endif
 
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB>
 __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
-    typedef RingGeo<D, QT> R;
+    typedef RingGeo<D, QT, KB> R;
     static_assert(R::TPW >= 1 && R::Q_BYTES % 1024 == 0, "query slab too small for this head dim");
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
     constexpr int C = R::C, BKV = R::BKV, TPB = R::TPB, TPW = R::TPW, RP = R::RP, KQ = R::KQ, QR = R::QR;
@@ -492,11 +494,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB>
 static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    typedef RingGeo<D, QT> R;
+    typedef RingGeo<D, QT, KB> R;
     static bool attr_set = false;
-    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT>;
+    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB>;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES) != hipSuccess)
             return EVO_EHIP;
@@ -509,31 +511,42 @@ static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 }
 
 // The forms the kernel is built in.  Per key tile of a row a wave keeps 16 registers of bias
-// and 16 of dBias sums, so rows of one key block run with two query tiles per workgroup (two
-// key tiles per wave); longer rows run with one query tile per workgroup (one key tile per
-// wave and block, up to three blocks: with more the spilled form is slower than the
-// one-workgroup-per-problem kernel), head dim 8 up to two blocks with two query tiles.
+// and 16 of dBias sums (three tiles per wave fit, four spill and run slower than the
+// one-workgroup-per-problem kernel):
+//   head dims 8, 16, 32   N <= 256        1 block of 256 keys, 2 query tiles per workgroup (2 tiles per wave)
+//   head dim 8            N <= 512        2 blocks of 256 keys, 2 query tiles               (4 tiles per wave; its working set is small)
+//   head dims 16, 32      N <= 384        3 blocks of 128 keys, 2 query tiles               (3 tiles per wave; measured
+//                                         196 us against 256 us for the next form at N = 384, D = 32, S = 384, H = 4)
+//                         N <= 512, 768   2, 3 blocks of 256 keys, 1 query tile             (2, 3 tiles per wave)
+//   head dim 64           N <= 128        1 block of 128 keys, 2 query tiles                (1 tile per wave)
+struct DqrForm {
+    int nblk, qt, kb;   // nblk = 0: not built for such rows
+};
 template <int D>
-constexpr int dqr_key_blocks(int n) { return (n + RingGeo<D, 2>::BKV - 1) / RingGeo<D, 2>::BKV; }
-template <int D>
-constexpr int dqr_query_tiles(int n) {
-    const int nblk = dqr_key_blocks<D>(n);
-    if (nblk == 1) return 2;
-    if (D == 8) return nblk == 2 ? 2 : 0;
-    if (D == 16 || D == 32) return nblk <= 3 ? 1 : 0;
-    return 0;
+constexpr DqrForm dqr_form(int n) {
+    if (D == 64) return n <= 128 ? DqrForm{1, 2, 128} : DqrForm{0, 0, 0};
+    if (n <= 256) return DqrForm{1, 2, 256};
+    if (D == 8) return n <= 512 ? DqrForm{2, 2, 256} : DqrForm{0, 0, 0};
+    if (n <= 384) return DqrForm{3, 2, 128};
+    if (n <= 512) return DqrForm{2, 1, 256};
+    if (n <= 768) return DqrForm{3, 1, 256};
+    return DqrForm{0, 0, 0};
 }
 
 template <typename T, int D, bool HAS_BIAS>
 static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const int nblk = dqr_key_blocks<D>(p.N);
-    if (nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2>(p, e, st);
-    if constexpr (D == 8) {
-        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 2>(p, e, st);
-    }
-    if constexpr (D == 16 || D == 32) {
-        if (nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 1>(p, e, st);
-        if (nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3, 1>(p, e, st);
+    const DqrForm f = dqr_form<D>(p.N);
+    if constexpr (D == 64) {
+        if (f.nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2, 128>(p, e, st);
+    } else {
+        if (f.nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2, 256>(p, e, st);
+        if constexpr (D == 8) {
+            if (f.nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 2, 256>(p, e, st);
+        } else {
+            if (f.nblk == 3 && f.kb == 128) return dqr_launch<T, D, HAS_BIAS, 3, 2, 128>(p, e, st);
+            if (f.nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 1, 256>(p, e, st);
+            if (f.nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3, 1, 256>(p, e, st);
+        }
     }
     return EVO_EUNSUPPORTED;
 }
@@ -545,7 +558,7 @@ static int dqr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 
 // Query rows one workgroup of the double-buffered dQ kernel takes at this N (64 or 32); 0
 // where the kernel is not built for such rows.
-int EVO_CAT(mfma_dqr_qrows_d, EVO_D)(int n) { return 32 * dqr_query_tiles<EVO_D>(n); }
+int EVO_CAT(mfma_dqr_qrows_d, EVO_D)(int n) { return 32 * dqr_form<EVO_D>(n).qt; }
 
 int EVO_CAT(launch_mfma_dqr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.dtype == EVO_BF16 ? dqr_bias<bf16_t, EVO_D>(p, e, st) : dqr_bias<f16_t, EVO_D>(p, e, st);
