@@ -49,6 +49,30 @@ __device__ __forceinline__ uint2 ones3() {
     return __builtin_bit_cast(uint2, v);
 }
 
+// Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
+// copy of the kernel) and reports that device's CU count.  `done` is the caller's per-kernel
+// state, one slot per device ordinal.
+constexpr int kMaxDevices = 64;
+struct PerDevice {
+    bool set[kMaxDevices];
+    int cus[kMaxDevices];
+};
+static inline int ensure_dynamic_lds(const void *kern, int bytes, PerDevice &done, int *cus) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
+    if (dev < 0 || dev >= kMaxDevices) return EVO_EUNSUPPORTED;
+    if (!done.set[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        const hipError_t err = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (err != hipSuccess) return EVO_EHIP - (int)err;
+        done.cus[dev] = n;
+        done.set[dev] = true;
+    }
+    if (cus) *cus = done.cus[dev];
+    return EVO_OK;
+}
+
 static inline int hip_rc() {
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;

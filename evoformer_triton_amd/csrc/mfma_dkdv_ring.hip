@@ -368,17 +368,10 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
 template <typename T, int D, bool HAS_BIAS>
 static int kvr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
     typedef KvRingGeo<D> R;
-    static int cus = 0;
-    static bool attr_set = false;
+    static PerDevice done{};
+    int cus = 256;
     auto kern = mfma_dkdv_ring<T, D, HAS_BIAS>;
-    if (!attr_set) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        hipError_t err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES);
-        if (err != hipSuccess) return EVO_EHIP - (int)err;
-        attr_set = true;
-    }
+    if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, &cus)) return rc;
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     // (these chunks are the kernel's own; the dBias partials keep theirs)
     Extra e = e0;

@@ -497,13 +497,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB>
 static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     typedef RingGeo<D, QT, KB> R;
-    static bool attr_set = false;
+    static PerDevice done{};
     auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB>;
-    if (!attr_set) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES) != hipSuccess)
-            return EVO_EHIP;
-        attr_set = true;
-    }
+    if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, nullptr)) return rc;
     const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
     const unsigned grid = (unsigned)NQP * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
     kern<<<grid, 512, R::LDS_BYTES, st>>>(p, e);

@@ -476,17 +476,10 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 template <typename T, int D, int BIASK>
 static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
     typedef FwdRingGeo<D> R;
-    static int cus = 0;
-    static bool attr_set = false;
+    static PerDevice done{};
+    int cus = 256;
     auto kern = mfma_fwd_ring<T, D, BIASK>;
-    if (!attr_set) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        hipError_t err = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, R::LDS_BYTES);
-        if (err != hipSuccess) return EVO_EHIP - (int)err;
-        attr_set = true;
-    }
+    if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, &cus)) return rc;
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     Extra e = e0;
     const int bh = p.B * p.H;
