@@ -156,6 +156,68 @@ def test_c_abi_direct_call_with_lse(E):
     assert lib.evoattn_bwd(ctypes.byref(p), st) == _lib.EVO_EWORKSPACE
 
 
+def test_c_abi_under_graph_capture(E):
+    """The entry points allocate nothing, synchronise nothing and use only the stream they are given,
+    so a forward+backward can be captured into a graph: replays (with eager work and fresh inputs
+    between them) give what the direct calls give."""
+    import ctypes
+    from evoformer_triton_amd import _lib
+    lib = _lib.load()
+    B, S, N, H, D = 1, 24, 256, 2, 32        # the kernels that walk over a chunk of S rows
+    dev = "cuda"
+    g = torch.Generator().manual_seed(21)
+    mk = lambda *shape: torch.randn(shape, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, dO = mk(B, S, N, H, D), mk(B, S, N, H, D), mk(B, S, N, H, D), mk(B, S, N, H, D)
+    bias = (mk(B, H, N, N) * 0.5).contiguous()
+    mask = (torch.rand((B, S, N), generator=g) < 0.85).to(dev)
+    o, lse = torch.empty_like(q), torch.empty((B, H, S, N), device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    dbias = torch.empty((B, H, N, N), device=dev, dtype=torch.bfloat16)
+    p = _lib.EvoAttnParams()
+    p.B, p.S, p.N, p.H, p.D = B, S, N, H, D
+    p.dtype, p.bias_dtype, p.mask_kind, p.dbias_dtype = _lib.EVO_BF16, _lib.EVO_BF16, _lib.EVO_MASK_BOOL, _lib.EVO_BF16
+    p.scale = D ** -0.5
+    p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * H * D, S * N * D, N * D, D
+    p.bias_stride_b, p.bias_stride_h, p.bias_stride_row = H * N * N, N * N, N
+    p.mask_stride_b, p.mask_stride_s = S * N, N
+    for name, t in (("q", q), ("k", k), ("v", v), ("bias", bias), ("mask", mask), ("o", o), ("lse", lse),
+                    ("dout", dO), ("dq", dq), ("dk", dk), ("dv", dv), ("dbias", dbias)):
+        setattr(p, name, t.data_ptr())
+    prep = torch.empty(lib.evoattn_prep_bytes(ctypes.byref(p)), dtype=torch.uint8, device=dev)
+    p.prep, p.prep_bytes = prep.data_ptr(), prep.numel()
+    ws = torch.empty(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), dtype=torch.uint8, device=dev)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    assert lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD) == b"mfma_dq_ring,mfma_dkdv_ring"
+
+    def run(stream):
+        st = ctypes.c_void_p(stream.cuda_stream)
+        p.flags = 0
+        assert lib.evoattn_fwd(ctypes.byref(p), st) == 0
+        p.flags = _lib.EVO_FLAG_PREP_VALID
+        assert lib.evoattn_bwd(ctypes.byref(p), st) == 0
+
+    outs = (o, lse, dq, dk, dv, dbias)
+    run(torch.cuda.current_stream())          # first use of the kernels outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run(torch.cuda.current_stream())
+    for rep in range(3):
+        for t in (q, k, v, dO):
+            t.copy_(torch.randn(t.shape, generator=g).to(torch.bfloat16))      # eager work between the replays
+        for t in outs:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        for t in outs:
+            t.zero_()
+        run(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        for a, b in zip(got, outs):
+            assert torch.equal(a, b), rep
+
+
 # ------------------------------------------------------------------ small seeded cases vs the CPU oracle
 
 SMALL = [
