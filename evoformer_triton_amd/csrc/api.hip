@@ -294,11 +294,14 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     const bool ring = dq_ring_ok(*p);
     if (p->flags & EVO_FLAG_ONLY_DQ) return ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st);
     const bool kvring = kv_ring_ok(*p);
+    // that kernel sums the dBias partials on its way in (they lie 16-byte aligned for it)
+    const bool fused_reduce = kvring && p->dbias && !(p->flags & EVO_FLAG_ONLY_DQ) && aligned(p->dbias, 16);
+    e.dbias_chunks = fused_reduce ? e.n_chunks : 0;
     if (p->flags & EVO_FLAG_ONLY_DKDV) return kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads
     if ((rc = ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st))) return rc;
     if ((rc = kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st))) return rc;
-    if (p->dbias && (rc = launch_dbias_reduce(*p, e, st))) return rc;
+    if (p->dbias && !fused_reduce && (rc = launch_dbias_reduce(*p, e, st))) return rc;
     if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;
     return EVO_OK;
 }

@@ -37,6 +37,7 @@ struct Extra {
     int vec_ok;        // bias rows may be read with 8/16-byte vector loads
     int bias_batches;  // 1 when one bias is shared by the whole batch, else B
     int bias_direct;   // the one-workgroup-per-problem kernels read the bias from the caller's tensor, not from bq / bk
+    int dbias_chunks;  // > 0: the dK/dV kernel over a chunk of rows also sums that many dBias partials (else `dbias_reduce` does)
     float *delta;      // [B][H][S][N]
     float *shift;      // [B][S] per-row mask shift (plain kernels)
     float *dbias_part; // [n_chunks][B][H][N][N]
