@@ -294,6 +294,12 @@ def main():
 
     esz = qc.element_size()
     io_bytes = 12 * qc.numel() * esz + 2 * bias.numel() * bias.element_size()   # algorithmic HBM bytes per step
+    # Algorithmic HBM bytes of each launch taken alone: every tensor it needs once.
+    t_b, l_b, b_b = qc.numel() * esz, lse.numel() * 4, bias.numel() * bias.element_size()
+    phase_bytes = {"fwd": 4 * t_b + l_b + b_b,                  # Q,K,V -> O, LSE
+                   "bwd_dq": 6 * t_b + 2 * l_b + 2 * b_b,       # Q,K,V,dO,O,LSE -> dQ, delta, dBias
+                   "bwd_dkdv": 6 * t_b + 2 * l_b + b_b}         # Q,K,V,dO,LSE,delta -> dK,dV
+    hbm_gbs = phase_bytes[dom] / t_phase[dom] / 1e9
     out = {
         "metric": "fwd+bwd TFLOP/s (S=%d N=%d H=%d D=%d)" % (S, N, H, D),
         "value": f_full / dt / 1e12,
@@ -321,7 +327,11 @@ def main():
         "roofline": {"bound": "mfma", "kernel": kernel_names[dom], "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
                      "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, kernel_names[dom].split("+")[-1])),
-                     "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3},
+                     "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3,
+                     # the same launch against the other ceiling: by intensity (flops / bytes below
+                     # peak flops / peak bytes) the memory ceiling is the lower of the two here
+                     "hbm": {"achieved": hbm_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": hbm_gbs / HBM_PEAK_GBS, "bytes_per_launch": phase_bytes[dom]}},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.config, (B, S, N, H, D))
