@@ -77,6 +77,20 @@ static bool dq_ring_ok(const EvoAttnParams &p) {
     return !(p.flags & EVO_FLAG_PER_PROBLEM) && !bias_direct(p) && mfma_dqr_qrows(p.D, p.N) > 0;
 }
 
+// Where dBias is not a sum over S rows (no bias, one that takes no gradient, or S = 1, where
+// dBias is dS itself) nothing ties a wave of the dQ kernel to a key tile for a chunk of S rows:
+// the kernel whose waves own their query rows for all keys takes those problems, and with
+// S = 1 writes dBias as it goes (no partials, no reduction).  Bit 0x1000 of flags (not part of
+// the public interface) selects the other kernels, for comparison.
+static bool dq_wide_ok(const EvoAttnParams &p) {
+    if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x1000)) || (p.dbias && p.S != 1)) return false;
+    // its workgroups take 128 query rows each and walk over the keys one tile after the other:
+    // with very few of them the kernels that split a row's keys over the waves finish sooner
+    // (N = 300, 6 workgroups: 10.4 us against 8.2 us)
+    return (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
+}
+static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && dq_wide_ok(p); }
+
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
 // writes one partial dBias tile.  Enough chunks to fill the chip, no more.  The kernel that
 // walks over its chunk with one workgroup per CU (256 CUs) wants the workgroups to come in
@@ -163,7 +177,7 @@ static WsLayout ws_layout(const EvoAttnParams &p) {
     w.dmask_part = off; if (p.dmask) off += align_up(rows * 4);
     chunking(p, &w.n_chunks, &w.chunk);
     w.dbias_part = off;
-    if (p.dbias) off += align_up((size_t)w.n_chunks * p.B * p.H * p.N * p.N * 4);
+    if (p.dbias && !dq_writes_dbias(p)) off += align_up((size_t)w.n_chunks * p.B * p.H * p.N * p.N * 4);
     w.total = off;
     return w;
 }
@@ -249,11 +263,18 @@ static bool kv_ring_ok(const EvoAttnParams &p) {
     return !p.bias || p.bias_dtype == p.dtype;
 }
 
+static int launch_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    if (dq_wide_ok(p)) return launch_mfma_dqw(p, e, st);
+    return dq_ring_ok(p) ? launch_mfma_dqr(p, e, st) : launch_mfma_dq(p, e, st);
+}
+
 const char *evoattn_kernels(const EvoAttnParams *p, int pass) {
     if (!p) return "invalid";
     if (!mfma_ok(*p, pass)) return "generic";
     if (pass == EVO_PASS_FWD) return fwd_ring_ok(*p) ? "mfma_fwd_ring" : "mfma_fwd";
-    if (kv_ring_ok(*p)) return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv_ring" : "mfma_dq,mfma_dkdv_ring";
+    const bool kvr = kv_ring_ok(*p);
+    if (dq_wide_ok(*p)) return kvr ? "mfma_dq_wide,mfma_dkdv_ring" : "mfma_dq_wide,mfma_dkdv";
+    if (kvr) return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv_ring" : "mfma_dq,mfma_dkdv_ring";
     return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv" : "mfma_dq,mfma_dkdv";
 }
 
@@ -291,17 +312,17 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
     fill_prep(*p, e);
     EVO_SET_TRACE(e);
     if (!(p->flags & EVO_FLAG_PREP_VALID) && (rc = launch_prep(*p, e, st))) return rc;
-    const bool ring = dq_ring_ok(*p);
-    if (p->flags & EVO_FLAG_ONLY_DQ) return ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st);
+    if (p->flags & EVO_FLAG_ONLY_DQ) return launch_dq(*p, e, st);
     const bool kvring = kv_ring_ok(*p);
     // that kernel sums the dBias partials on its way in (they lie 16-byte aligned for it)
-    const bool fused_reduce = kvring && p->dbias && !(p->flags & EVO_FLAG_ONLY_DQ) && aligned(p->dbias, 16);
+    const bool partials = p->dbias && !dq_writes_dbias(*p);
+    const bool fused_reduce = kvring && partials && !(p->flags & EVO_FLAG_ONLY_DQ) && aligned(p->dbias, 16);
     e.dbias_chunks = fused_reduce ? e.n_chunks : 0;
     if (p->flags & EVO_FLAG_ONLY_DKDV) return kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads
-    if ((rc = ring ? launch_mfma_dqr(*p, e, st) : launch_mfma_dq(*p, e, st))) return rc;
+    if ((rc = launch_dq(*p, e, st))) return rc;
     if ((rc = kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st))) return rc;
-    if (p->dbias && !fused_reduce && (rc = launch_dbias_reduce(*p, e, st))) return rc;
+    if (partials && !fused_reduce && (rc = launch_dbias_reduce(*p, e, st))) return rc;
     if (p->dmask && (rc = launch_dmask_reduce(*p, e, st))) return rc;
     return EVO_OK;
 }

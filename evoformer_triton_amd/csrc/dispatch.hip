@@ -13,7 +13,8 @@ namespace evo {
     int mfma_dqr_qrows_d##D(int);                                                            \
     int launch_mfma_kvr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
     int mfma_kvr_max_n_d##D();                                                               \
-    int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
+    int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);            \
+    int launch_mfma_dqw_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
 EVO_DECL(16)
 EVO_DECL(32)
@@ -36,6 +37,7 @@ EVO_ROUTE(dq)
 EVO_ROUTE(dqr)
 EVO_ROUTE(kvr)
 EVO_ROUTE(dkdv)
+EVO_ROUTE(dqw)
 #undef EVO_ROUTE
 
 int mfma_fwdr_max_n(int D) {

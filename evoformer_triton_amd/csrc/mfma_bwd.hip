@@ -340,7 +340,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 #endif
 
 template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
-__global__ void __launch_bounds__(NW * 64, NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
+__global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef KvGeo<D> R;
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;

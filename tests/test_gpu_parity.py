@@ -340,6 +340,99 @@ def test_bias_read_from_the_callers_tensor_matches_the_prepared_tiles(E, shape, 
         assert torch.equal(a[name], b[name]), (name, max_err(a[name], b[name]))
 
 
+# B, S, N, H, D, mask, bias ("q": bias in the dtype of q that takes no gradient), dtype
+NO_DBIAS = [
+    (1, 40, 256, 2, 32, "add", None, torch.bfloat16),
+    (2, 20, 130, 2, 8, "bool", None, torch.bfloat16),
+    (1, 12, 520, 3, 64, "soft", None, torch.float16),
+    (1, 33, 200, 1, 16, "bool", "q", torch.bfloat16),
+    (1, 9, 640, 2, 32, "add", "q", torch.bfloat16),
+    (1, 64, 100, 1, 64, None, None, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", NO_DBIAS, ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_dq_where_no_dbias_is_asked_for(E, case):
+    """Without a pair bias, or with one that takes no gradient, dQ comes from the kernel whose
+    waves own their query rows for all keys (`evoattn_kernels` names it); checked against the CPU
+    oracle in fp32 and, to a 16-bit unit in the last place, against the kernels that split the keys
+    over the waves (flag bit 0x1000)."""
+    B, S, N, H, D, mask, bias_dt, dtype = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, dtype, seed=11)
+    if m is not None and S > 2 and (m.dtype == torch.bool or dtype == torch.bfloat16):
+        m[:, 1] = False if m.dtype == torch.bool else -1e9      # a row with every key masked (-1e9 is -inf in fp16)
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
+
+    def run(flags):
+        q, k, v = (t.cuda().requires_grad_() for t in (Q, K, V))
+        b = None if bias is None else bias.cuda()              # no requires_grad: no dBias
+        try:
+            E.FLAGS = flags
+            o = E.evoformer_attention(q, k, v, None if m is None else m.cuda(), b)
+            o.backward(dO.cuda())
+        finally:
+            E.FLAGS = 0
+        torch.cuda.synchronize()
+        return {"O": o.detach(), "dQ": q.grad, "dK": k.grad, "dV": v.grad}
+
+    got, other = run(0), run(0x1000)
+    assert_close(got, ref, BF16_TOL if dtype == torch.bfloat16 else 4e-3, ["O", "dQ", "dK", "dV"], what=str(case))
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for name in got:
+        assert max_err(got[name], other[name]) <= ulp * max(1.0, other[name].abs().max().item()), name
+
+
+def test_dq_kernel_choice_is_reported(E):
+    """`evoattn_kernels` names the dQ kernel that a call would launch: the one without a sum over
+    S rows where no dBias is asked for or S = 1, given enough workgroups."""
+    from evoformer_triton_amd import _lib
+    lib = _lib.load()
+
+    def kernels(shape, with_bias, with_dbias, flags=0):
+        B, S, N, H, D = shape
+        q = torch.empty((B, S, N, H, D), device="cuda", dtype=torch.bfloat16)
+        bias = torch.empty((B, 1, H, N, N), device="cuda", dtype=torch.bfloat16) if with_bias else None
+        mask, mk, mstr = E._prep_mask(None, B, S, N, q.device)
+        bz, bdt, bstr = E._prep_bias(bias, B, H, N, q.dtype, q.device)
+        lse = torch.empty((B, H, S, N), device="cuda")
+        p = E._params(q, q, q, mask, mk, mstr, bz, bdt, bstr, q, lse, "reference")
+        if with_dbias:
+            p.dbias, p.dbias_dtype = bz.data_ptr(), E._DTYPES[torch.bfloat16]
+        p.flags = flags
+        return lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().split(",")[0]
+
+    assert kernels((1, 64, 256, 4, 32), False, False) == "mfma_dq_wide"
+    assert kernels((1, 64, 256, 4, 32), True, False) == "mfma_dq_wide"
+    assert kernels((1, 64, 256, 4, 32), True, True) == "mfma_dq_ring"
+    assert kernels((4, 1, 512, 8, 64), True, True) == "mfma_dq_wide"          # S = 1: dBias is dS
+    assert kernels((4, 1, 512, 8, 64), True, True, 0x1000) == "mfma_dq"
+    assert kernels((1, 2, 300, 1, 64), False, False) == "mfma_dq"             # six workgroups: keys split over waves
+
+
+@pytest.mark.parametrize("case", [(4, 1, 256, 8, 64, "q", torch.bfloat16), (2, 1, 200, 16, 32, torch.float32, torch.bfloat16),
+                                  (8, 1, 130, 4, 16, "q", torch.float16), (3, 1, 513, 4, 8, "q", torch.bfloat16)],
+                         ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_single_row_problems_write_dbias_from_the_dq_kernel(E, case):
+    """S = 1 (the shape of the reference's speed_benchmark.py): dBias of a (batch, head) is the dS
+    of its one row; the dQ kernel writes it as it goes, no partial sums, no reduction.  Checked
+    against the CPU oracle, and the workspace no longer holds an fp32 copy of dBias."""
+    from evoformer_triton_amd import _lib
+    B, S, N, H, D, bias_dt, dtype = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, "bool", bias_dt, dtype, seed=13)
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
+    got = run_hip(E, Q, K, V, m, bias, dO)
+    assert_close(got, ref, BF16_TOL if dtype == torch.bfloat16 else 4e-3, what=str(case))
+    lib = _lib.load()
+    q = Q.cuda()
+    mask, mk, mstr = E._prep_mask(m.cuda(), B, S, N, q.device)
+    bz, bdt, bstr = E._prep_bias(bias.cuda(), B, H, N, q.dtype, q.device)
+    lse = torch.empty((B, H, S, N), device="cuda")
+    p = E._params(q, q, q, mask, mk, mstr, bz, bdt, bstr, q, lse, "reference")
+    p.dbias, p.dbias_dtype = bz.data_ptr(), E._DTYPES[bz.dtype]
+    assert lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().startswith("mfma_dq_wide")
+    assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) < B * H * N * N * 4
+
+
 def test_c1_fp32_check_mode_against_cpu_eager(E):
     x = eager.make_inputs("C1")
     ref = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"])     # fp32, as specified
