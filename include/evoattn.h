@@ -148,7 +148,7 @@ int evoattn_bwd(const EvoAttnParams *p, void *hip_stream);
 const char *evoattn_path(const EvoAttnParams *p, int pass);
 
 /* Names of the main kernels that pass would launch, comma separated (e.g. "mfma_fwd_ring",
- * "mfma_dq_ring,mfma_dkdv", "generic"); for reports and profiles. */
+ * "mfma_dq_ring,mfma_dkdv", "mfma_dq_wide,mfma_dkdv", "generic"); for reports and profiles. */
 const char *evoattn_kernels(const EvoAttnParams *p, int pass);
 
 #ifdef __cplusplus
