@@ -309,10 +309,10 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 // row-major: Q pre-multiplied by scale*log2(e) exactly as in the forward, dO, and per query the
 // 16-bit columns that carry -LSE and -delta into the score MFMAs.  The transposed operands
 // of dV^T += dO^T P and dK^T += Q^T dS come from the same rows by transposing LDS reads
-// (`ds_read_b64_tr_b16`).  For head dims <= 16 the scaled Q is staged with its rounding residue
-// (as the scores need it), dK sums over both and is multiplied by scale / (scale*log2(e)) = ln 2
-// at the end; for the larger head dims Q is staged a second time as given and dK is
-// multiplied by scale (summing over the rounded scaled Q alone costs dK two digits at N = 768).
+// (`ds_read_b64_tr_b16`).  Q is staged a second time as given: dK sums over that copy and is
+// multiplied by scale at the end (summing over the rounded scaled Q alone costs dK two digits
+// at N = 768); for head dims <= 16 the rounding residue of the scaled Q is staged as well, for
+// the scores only (a third set of transposing reads and twice the dK MFMAs if dK used it).
 // Scores are NOT transposed here: a lane owns one key and 16 queries, so that P and dS in
 // accumulator layout are the B operands of the two gradient matmuls.
 template <int D>
@@ -322,8 +322,8 @@ struct KvGeo {
     static constexpr int BQS = D <= 32 ? 256 : 128;          // query rows staged per round
     static constexpr bool RESID = D <= 16;
     // LDS layout for `rows` staged query rows (BQS, or 128 where a problem has no more):
-    //   [Q scaled][its rounding residue (RESID) or Q as given][dO][-LSE columns][-delta columns]
-    static __host__ __device__ constexpr int lds_bytes(int rows) { return rows * (3 * D * 2 + 32); }
+    //   [Q scaled][Q as given][dO]([rounding residue of Q scaled] for RESID)[-LSE columns][-delta columns]
+    static __host__ __device__ constexpr int lds_bytes(int rows) { return rows * ((RESID ? 4 : 3) * D * 2 + 32); }
     static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
 };
 
@@ -360,8 +360,9 @@ __global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nkb = (p.N + BK - 1) / BK;
     constexpr int srows = BQS;
-    constexpr int OFF_QS = 0, OFF_QL = srows * D * 2, OFF_QR = OFF_QL, OFF_G = 2 * OFF_QL;
-    constexpr int OFF_AQ = 3 * OFF_QL, OFF_AG = OFF_AQ + srows * 16;
+    constexpr int BLK = srows * D * 2;
+    constexpr int OFF_QS = 0, OFF_QR = BLK, OFF_G = 2 * BLK, OFF_QL = 3 * BLK;
+    constexpr int OFF_AQ = (R::RESID ? 4 : 3) * BLK, OFF_AG = OFF_AQ + srows * 16;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nkb;
     const int key0 = (lid % nkb) * BK + wave * 32;
@@ -449,8 +450,9 @@ __global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
                 scaled_hilo8<T>(a, cs, hi, lo);
                 const int o = R::swz(row, ch);
                 *reinterpret_cast<v8 *>(lds + OFF_QS + o) = hi;
-                *reinterpret_cast<v8 *>(lds + OFF_QL + o) = R::RESID ? lo : a;
+                *reinterpret_cast<v8 *>(lds + OFF_QR + o) = a;
                 *reinterpret_cast<v8 *>(lds + OFF_G + o) = bb2;
+                if (R::RESID) *reinterpret_cast<v8 *>(lds + OFF_QL + o) = lo;
             }
         }
         for (int row = tid; row < srows; row += NTH) {
@@ -539,7 +541,7 @@ __global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
             for (int dt = 0; dt < DT; ++dt) {
                 // dO^T and Q^T fragments: row d = dt*32 + li, the 8 queries the P registers hold
                 const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                v8 gta = zero8<T>(), qta = zero8<T>(), qtl = zero8<T>();
+                v8 gta = zero8<T>(), qta = zero8<T>();
                 if (col < D) {
 #pragma unroll
                     for (int h2 = 0; h2 < 2; ++h2) {
@@ -548,25 +550,17 @@ __global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
                         s16x4 rg = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                             (s16x4 __attribute__((address_space(3))) *)(lds + OFF_G + o));
                         s16x4 rq = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (s16x4 __attribute__((address_space(3))) *)(lds + (R::RESID ? OFF_QS : OFF_QR) + o));
+                            (s16x4 __attribute__((address_space(3))) *)(lds + OFF_QR + o));
                         v4 vg = __builtin_bit_cast(v4, rg), vq = __builtin_bit_cast(v4, rq);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             gta[4 * h2 + i] = vg[i];
                             qta[4 * h2 + i] = vq[i];
                         }
-                        if (R::RESID) {
-                            s16x4 rl = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                (s16x4 __attribute__((address_space(3))) *)(lds + OFF_QL + o));
-                            v4 vl = __builtin_bit_cast(v4, rl);
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) qtl[4 * h2 + i] = vl[i];
-                        }
                     }
                 }
                 dv[dt] = Mfma<T>::mma(gta, pf, dv[dt]);
                 dk[dt] = Mfma<T>::mma(qta, dsf, dk[dt]);
-                if (R::RESID) dk[dt] = Mfma<T>::mma(qtl, dsf, dk[dt]);
             }
         }
     };
@@ -606,8 +600,7 @@ __global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
         if (key < p.N) {
             T *dK = (T *)p.dk + pr.base + (int64_t)key * sn;
             T *dV = (T *)p.dv + pr.base + (int64_t)key * sn;
-            // with the residue, dk holds the sum over Q * scale * log2(e)
-            const float kscale = R::RESID ? kLn2 : p.scale;
+            const float kscale = p.scale;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 store_row_tile<T>(dK, dt * 32, D, dk[dt], kscale, g);
