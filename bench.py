@@ -37,6 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # inside this script, so only the profiled workload has a figure.
 MEASURED_HBM_BYTES_PER_LAUNCH = {
     ("C2", "mfma_fwd_ring"): 295.4e6, ("C2", "mfma_dq_ring"): 446.9e6, ("C2", "mfma_dkdv_ring"): 450.4e6,
+    ("C2-nobias", "mfma_fwd_ring"): 289.6e6, ("C2-nobias", "mfma_dq_wide"): 419.5e6, ("C2-nobias", "mfma_dkdv_ring"): 430.3e6,
 }
 
 
@@ -51,6 +52,9 @@ def parse():
                          "takes some tenths of a second of load to reach its steady clocks, and a handful of "
                          "400-microsecond warm-up steps ends before that (measured: 8 % slower steps)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-bias", action="store_true",
+                    help="the same shape without the pair bias (and so without dBias): the no-bias forms of the "
+                         "kernels, e.g. for a profile of them; not the headline workload")
     ap.add_argument("--reference-sweep", action="store_true",
                     help="instead of the step benchmark: the reference's own speed benchmark (speed_benchmark.py:37-115: "
                          "B=4, H=32, D=64, N_seq=1, bool mask, fp32 pair bias, modes fwd / bwd / full, timed like "
@@ -151,7 +155,7 @@ def reference_sweep():
                                           "peak_memory_bf16_bias": mem}}))
 
 
-def cpu_baseline(cfg, shape, budget_s=15.0):
+def cpu_baseline(cfg, shape, budget_s=15.0, with_bias=True):
     """The eager oracle (fp32, chunked over S) on the host cores, on a slice of S rows."""
     import torch
     from oracle import eager
@@ -162,7 +166,7 @@ def cpu_baseline(cfg, shape, budget_s=15.0):
 
     def once():
         t0 = time.perf_counter()
-        eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"],
+        eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"] if with_bias else None, x["dO"],
                                 compute_dtype=torch.float32, s_chunk=8)
         return time.perf_counter() - t0
 
@@ -194,13 +198,13 @@ def main():
     x = eager.make_inputs(args.config)
     B, S, N, H, D = x["shape"]
     q, k, v = (x[n].to(dev).requires_grad_() for n in "QKV")
-    bias = x["bias"].to(dev).requires_grad_()
+    bias = None if args.no_bias else x["bias"].to(dev).requires_grad_()
     mask, dO = x["mask"].to(dev), x["dO"].to(dev)
     f_fwd, f_bwd, f_full = eager.flops_fwd_bwd(B, S, N, H, D)
 
     def step():
         o = EvoformerAttention.apply(q, k, v, mask, bias)
-        return torch.autograd.grad(o, (q, k, v, bias), dO)
+        return torch.autograd.grad(o, (q, k, v) if bias is None else (q, k, v, bias), dO)
 
     t_heat = time.perf_counter()
     while time.perf_counter() - t_heat < args.preheat_seconds:
@@ -222,16 +226,17 @@ def main():
     # ---- kernel-level timing through the C ABI, buffers preallocated
     qc, kc, vc = q.detach(), k.detach(), v.detach()
     m, mk, mstr = E._prep_mask(mask, B, S, N, dev)
-    bz, bdt, bstr = E._prep_bias(bias.detach(), B, H, N, qc.dtype, dev)
+    bz, bdt, bstr = E._prep_bias(None if bias is None else bias.detach(), B, H, N, qc.dtype, dev)
     o = torch.empty_like(qc)
     lse = torch.empty((B, H, S, N), device=dev)
     p = E._params(qc, kc, vc, m, mk, mstr, bz, bdt, bstr, o, lse, "reference")
     prep = E._alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), dev)
     p.prep, p.prep_bytes = prep.data_ptr(), prep.numel()
     dq, dk, dv = (torch.empty_like(qc) for _ in range(3))
-    dbias = torch.empty((B, H, N, N), device=dev, dtype=bz.dtype)
-    p.dout, p.dq, p.dk, p.dv, p.dbias = dO.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dbias.data_ptr()
-    p.dbias_dtype = E._DTYPES[bz.dtype]
+    p.dout, p.dq, p.dk, p.dv = dO.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    if bz is not None:
+        dbias = torch.empty((B, H, N, N), device=dev, dtype=bz.dtype)
+        p.dbias, p.dbias_dtype = dbias.data_ptr(), E._DTYPES[bz.dtype]
     ws = E._alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), dev)
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -293,9 +298,10 @@ def main():
         torch.cuda.synchronize()
 
     esz = qc.element_size()
-    io_bytes = 12 * qc.numel() * esz + 2 * bias.numel() * bias.element_size()   # algorithmic HBM bytes per step
+    b_b = 0 if bias is None else bias.numel() * bias.element_size()
+    io_bytes = 12 * qc.numel() * esz + 2 * b_b   # algorithmic HBM bytes per step
     # Algorithmic HBM bytes of each launch taken alone: every tensor it needs once.
-    t_b, l_b, b_b = qc.numel() * esz, lse.numel() * 4, bias.numel() * bias.element_size()
+    t_b, l_b = qc.numel() * esz, lse.numel() * 4
     phase_bytes = {"fwd": 4 * t_b + l_b + b_b,                  # Q,K,V -> O, LSE
                    "bwd_dq": 6 * t_b + 2 * l_b + 2 * b_b,       # Q,K,V,dO,O,LSE -> dQ, delta, dBias
                    "bwd_dkdv": 6 * t_b + 2 * l_b + b_b}         # Q,K,V,dO,LSE,delta -> dK,dV
@@ -315,7 +321,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.config}: Evoformer attention fwd+bwd through EvoformerAttention.apply + autograd, "
                                f"Q,K,V [B={B},S={S},N={N},H={H},D={D}] bf16, additive row mask [{B},{S},1,1,{N}], "
-                               f"pair bias [{B},1,{H},{N},{N}] bf16, seeded N(0,1) inputs",
+                               + ("no pair bias" if bias is None else f"pair bias [{B},1,{H},{N},{N}] bf16") + ", seeded N(0,1) inputs",
                    "flops_per_step": f_full, "algorithmic_hbm_bytes_per_step": io_bytes},
         "pct_mfma_peak": 100.0 * f_full / dt / 1e12 / MFMA_PEAK_TFLOPS,
         "pct_hbm_peak": 100.0 * io_bytes / dt / 1e9 / HBM_PEAK_GBS,
@@ -326,7 +332,8 @@ def main():
         "peak_mem_bytes_beyond_inputs": int(peak_extra),
         "roofline": {"bound": "mfma", "kernel": kernel_names[dom], "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config, kernel_names[dom].split("+")[-1])),
+                     "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config + ("" if bias is not None else "-nobias"),
+                                                                    kernel_names[dom].split("+")[-1])),
                      "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3,
                      # the same launch against the other ceiling: by intensity (flops / bytes below
                      # peak flops / peak bytes) the memory ceiling is the lower of the two here
@@ -334,7 +341,7 @@ def main():
                              "frac": hbm_gbs / HBM_PEAK_GBS, "bytes_per_launch": phase_bytes[dom]}},
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.config, (B, S, N, H, D))
+        out["cpu_baseline"] = cpu_baseline(args.config, (B, S, N, H, D), with_bias=bias is not None)
     print(json.dumps(out))
 
 
