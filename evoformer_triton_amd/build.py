@@ -44,6 +44,7 @@ def _units():
         units.append((f"mfma_dqr_d{d}", "mfma_dq_ring.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_kvr_d{d}", "mfma_dkdv_ring.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_dqw_d{d}", "mfma_dq_wide.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
+        units.append((f"mfma_dbias_d{d}", "mfma_dbias.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
     return units
 
 

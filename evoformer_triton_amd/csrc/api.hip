@@ -80,16 +80,32 @@ static bool dq_ring_ok(const EvoAttnParams &p) {
 // Where dBias is not a sum over S rows (no bias, one that takes no gradient, or S = 1, where
 // dBias is dS itself) nothing ties a wave of the dQ kernel to a key tile for a chunk of S rows:
 // the kernel whose waves own their query rows for all keys takes those problems, and with
-// S = 1 writes dBias as it goes (no partials, no reduction).  Bit 0x1000 of flags (not part of
-// the public interface) selects the other kernels, for comparison.
-static bool dq_wide_ok(const EvoAttnParams &p) {
-    if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x1000)) || (p.dbias && p.S != 1)) return false;
-    // its workgroups take 128 query rows each and walk over the keys one tile after the other:
-    // with very few of them the kernels that split a row's keys over the waves finish sooner
-    // (N = 300, 6 workgroups: 10.4 us against 8.2 us)
-    return (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
+// S = 1 writes dBias as it goes (no partials, no reduction).  Its workgroups take 128 query
+// rows each and walk over the keys one tile after the other: with very few of them the
+// kernels that split a row's keys over the waves finish sooner (N = 300, 6 workgroups: 10.4 us
+// against 8.2 us).  Bit 0x1000 of flags (not part of the public interface) selects the other
+// kernels, for comparison.
+static bool dq_wide_grid_ok(const EvoAttnParams &p) {
+    return !(p.flags & (EVO_FLAG_PER_PROBLEM | 0x1000)) && (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
 }
-static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && dq_wide_ok(p); }
+
+// Rows of more than 384 keys with a dBias to sum (up to there the dQ kernel that keeps the sums
+// has two query tiles per workgroup, beyond one): dQ from that same kernel, and the dBias
+// partials from a kernel of their own that forms dS a second time (dQ and partials, S = N:
+// N = 512: 436 against 483 us, N = 768: 1.32 against 1.67 ms, N = 1024, S = 256: 0.80 against
+// 1.56 ms; N = 384: 211 against 204 us, and with few S rows the second kernel's start-up shows;
+// head dims 8 and 16, whose one-kernel form reaches to N = 512: 569 against 367 us and 696
+// against 661 us there, 0.65 against 1.38 ms and 740 against 793 us at N = 768).
+// Bit 0x2000 of flags (not part of the public interface) selects the one kernel, for comparison.
+static bool dq_split_ok(const EvoAttnParams &p) {
+    if (!p.dbias || p.S < 64 || p.N <= (p.D == 32 ? 384 : 512) || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
+    return p.D <= 32 && p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs, in 32 registers
+}
+
+static bool dq_wide_ok(const EvoAttnParams &p) {
+    return dq_wide_grid_ok(p) && (!p.dbias || p.S == 1 || dq_split_ok(p));
+}
+static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && p.S == 1 && dq_wide_ok(p); }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
 // writes one partial dBias tile.  Enough chunks to fill the chip, no more.  The kernel that
@@ -98,6 +114,24 @@ static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && dq_wide_
 // leaves the fewest CUs idle in the last round (ties: the fewest chunks).
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t NT = (p.N + 31) / 32;
+    if (dq_split_ok(p)) {
+        // the dBias kernel: one workgroup per block of 128 queries x 128 keys, (b, h) and chunk, two
+        // workgroups per CU (256 CUs) at a time; among the chunk counts that give one to four rounds
+        // the one that leaves the fewest slots idle in the last round (near ties: the fewest chunks)
+        const int64_t nb = (p.N + 127) / 128, base = nb * nb * p.B * p.H, slots = 512;
+        const int64_t lo = (slots + base - 1) / base, hi = (4 * slots + base - 1) / base;
+        int64_t want = lo;
+        double best = -1.0;
+        for (int64_t n = lo; n <= hi; ++n) {
+            const int64_t wgs = base * n, rounds = (wgs + slots - 1) / slots;
+            const double eff = (double)wgs / (double)(rounds * slots);
+            if (eff > best + 0.02) { best = eff; want = n; }
+        }
+        if (want > p.S) want = p.S;
+        *chunk = (int)((p.S + want - 1) / want);
+        *n_chunks = (p.S + *chunk - 1) / *chunk;
+        return;
+    }
     const bool ring = dq_ring_ok(p);
     // workgroups per chunk: one per slab of query rows and head
     const int64_t base = (ring ? (p.N + mfma_dqr_qrows(p.D, p.N) - 1) / mfma_dqr_qrows(p.D, p.N) : NT) * p.B * p.H;
@@ -264,6 +298,12 @@ static bool kv_ring_ok(const EvoAttnParams &p) {
 }
 
 static int launch_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    if (dq_split_ok(p)) {
+        EvoAttnParams q = p;
+        q.dbias = nullptr;                       // dQ and delta first, then the dBias partials, which read delta
+        if (const int rc = launch_mfma_dqw(q, e, st)) return rc;
+        return launch_mfma_dbias(p, e, st);
+    }
     if (dq_wide_ok(p)) return launch_mfma_dqw(p, e, st);
     return dq_ring_ok(p) ? launch_mfma_dqr(p, e, st) : launch_mfma_dq(p, e, st);
 }
@@ -273,6 +313,7 @@ const char *evoattn_kernels(const EvoAttnParams *p, int pass) {
     if (!mfma_ok(*p, pass)) return "generic";
     if (pass == EVO_PASS_FWD) return fwd_ring_ok(*p) ? "mfma_fwd_ring" : "mfma_fwd";
     const bool kvr = kv_ring_ok(*p);
+    if (dq_split_ok(*p)) return kvr ? "mfma_dq_wide+mfma_dbias,mfma_dkdv_ring" : "mfma_dq_wide+mfma_dbias,mfma_dkdv";
     if (dq_wide_ok(*p)) return kvr ? "mfma_dq_wide,mfma_dkdv_ring" : "mfma_dq_wide,mfma_dkdv";
     if (kvr) return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv_ring" : "mfma_dq,mfma_dkdv_ring";
     return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv" : "mfma_dq,mfma_dkdv";

@@ -14,7 +14,8 @@ namespace evo {
     int launch_mfma_kvr_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
     int mfma_kvr_max_n_d##D();                                                               \
     int launch_mfma_dkdv_d##D(const EvoAttnParams &, const Extra &, hipStream_t);            \
-    int launch_mfma_dqw_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
+    int launch_mfma_dqw_d##D(const EvoAttnParams &, const Extra &, hipStream_t);             \
+    int launch_mfma_dbias_d##D(const EvoAttnParams &, const Extra &, hipStream_t);
 EVO_DECL(8)
 EVO_DECL(16)
 EVO_DECL(32)
@@ -38,6 +39,7 @@ EVO_ROUTE(dqr)
 EVO_ROUTE(kvr)
 EVO_ROUTE(dkdv)
 EVO_ROUTE(dqw)
+EVO_ROUTE(dbias)
 #undef EVO_ROUTE
 
 int mfma_fwdr_max_n(int D) {

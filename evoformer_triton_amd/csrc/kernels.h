@@ -24,5 +24,6 @@ int mfma_kvr_max_n(int D);  // largest N the chunk-of-rows dK/dV kernel takes (i
 int mfma_dqr_qrows(int D, int N);  // query rows per workgroup of the double-buffered dQ kernel (64 or 32), 0 where it is not built for such rows
 int launch_mfma_dkdv(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_mfma_dqw(const EvoAttnParams &p, const Extra &e, hipStream_t st);  // dQ where no dBias is asked for
+int launch_mfma_dbias(const EvoAttnParams &p, const Extra &e, hipStream_t st);  // dBias partials alone (reads delta)
 
 }  // namespace evo

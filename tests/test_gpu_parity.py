@@ -382,6 +382,40 @@ def test_dq_where_no_dbias_is_asked_for(E, case):
         assert max_err(got[name], other[name]) <= ulp * max(1.0, other[name].abs().max().item()), name
 
 
+@pytest.mark.parametrize("case", [(1, 64, 416, 1, 32, "add", torch.bfloat16), (1, 70, 520, 2, 16, "bool", torch.bfloat16),
+                                  (1, 64, 530, 1, 8, "soft", torch.float16), (2, 66, 400, 1, 32, "bool", torch.float16)],
+                         ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_long_rows_sum_dbias_in_a_kernel_of_its_own(E, case):
+    """Rows of more than 384 keys (512 at head dims 8 and 16) with at least 64 S rows: dQ from
+    the kernel whose waves own their query rows, the dBias partials from a second kernel that
+    forms dS again (`evoattn_kernels` names both).  Against the CPU oracle in fp32, and against
+    the one kernel that does both (flag bit 0x2000) to a 16-bit unit in the last place."""
+    from evoformer_triton_amd import _lib
+    B, S, N, H, D, mask, dtype = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, "q", dtype, seed=17)
+    if m.dtype == torch.bool or dtype == torch.bfloat16:
+        m[:, 3] = False if m.dtype == torch.bool else -1e9      # a row with every key masked
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
+    got = run_hip(E, Q, K, V, m, bias, dO)
+    try:
+        E.FLAGS = 0x2000
+        other = run_hip(E, Q, K, V, m, bias, dO)
+    finally:
+        E.FLAGS = 0
+    assert_close(got, ref, BF16_TOL if dtype == torch.bfloat16 else 4e-3, what=str(case))
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for name in got:
+        assert max_err(got[name], other[name]) <= ulp * max(1.0, other[name].abs().max().item()), name
+    lib = _lib.load()
+    q = Q.cuda()
+    mask_, mk, mstr = E._prep_mask(m.cuda(), B, S, N, q.device)
+    bz, bdt, bstr = E._prep_bias(bias.cuda(), B, H, N, q.dtype, q.device)
+    lse = torch.empty((B, H, S, N), device="cuda")
+    p = E._params(q, q, q, mask_, mk, mstr, bz, bdt, bstr, q, lse, "reference")
+    p.dbias, p.dbias_dtype = bz.data_ptr(), E._DTYPES[bz.dtype]
+    assert lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().startswith("mfma_dq_wide+mfma_dbias,")
+
+
 def test_dq_kernel_choice_is_reported(E):
     """`evoattn_kernels` names the dQ kernel that a call would launch: the one without a sum over
     S rows where no dBias is asked for or S = 1, given enough workgroups."""
