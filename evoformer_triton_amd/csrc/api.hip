@@ -119,7 +119,7 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
         // workgroups per CU (256 CUs) at a time; among the chunk counts that give one to four rounds
         // the one that leaves the fewest slots idle in the last round (near ties: the fewest chunks)
         const int64_t nb = (p.N + 127) / 128, base = nb * nb * p.B * p.H, slots = 512;
-        const int64_t lo = (slots + base - 1) / base, hi = (4 * slots + base - 1) / base;
+        const int64_t lo = slots / base > 0 ? slots / base : 1, hi = (4 * slots + base - 1) / base;
         int64_t want = lo;
         double best = -1.0;
         for (int64_t n = lo; n <= hi; ++n) {

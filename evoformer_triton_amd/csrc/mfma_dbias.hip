@@ -11,7 +11,8 @@
 // tiles, whose running sums (64 registers) and bias tiles (32, as 16-bit pairs) stay resident.  Per S row the
 // workgroup stages its 128 keys (K with the mask columns, V) in LDS, the waves fetch their own
 // query rows (Q, dO, LSE, delta, as written by the dQ kernel); both are requested one row ahead
-// into registers.  Per tile: two score MFMA chains, exp2, a multiply and 16 additions; no
+// into registers, and the keys go to the other of two LDS buffers after the row's tiles: one
+// barrier per row.  Per tile: two score MFMA chains, exp2, a multiply and 16 additions; no
 // conversions, no gradient matmul.  One partial per chunk; `dbias_reduce` adds them in order.
 #include "bwd_common.h"
 #include "kernels.h"
@@ -41,7 +42,7 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
     constexpr int NIT = (KB * C + NTH - 1) / NTH;            // 16-byte pieces of K (and of V) per thread and row
     typedef typename Mfma<T>::v8 v8;
 
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[R::LDS_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * R::LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, g = lane >> 5;
@@ -120,22 +121,29 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
         delta_n = e.delta[pr.row0 + qrow];
     };
 
-    fetch(s_begin);
-    for (int s = s_begin; s < s_end; ++s) {
-        const bool dead = e.dead[b * p.S + s] != 0;
-        const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
-        const float bscale = dead ? 0.0f : kLog2e;   // a row with every key masked takes no bias
-        __syncthreads();   // everybody is done with the keys of the row before
+    // keys of a row into the buffer of that row's parity
+    auto stash = [&](int buf) {
+        unsigned char *dst = lds + buf * R::LDS_BYTES;
 #pragma unroll
         for (int i = 0; i < NIT; ++i) {
             const int it = tid + i * NTH;
             if (it < KB * C) {
                 const int o = R::swz(it / C, it % C);
-                *reinterpret_cast<v8 *>(lds + R::OFF_K + o) = kv[i];
-                *reinterpret_cast<v8 *>(lds + R::OFF_V + o) = vv[i];
+                *reinterpret_cast<v8 *>(dst + R::OFF_K + o) = kv[i];
+                *reinterpret_cast<v8 *>(dst + R::OFF_V + o) = vv[i];
             }
         }
-        if (tid < KB) *reinterpret_cast<v8 *>(lds + R::OFF_AK + tid * 16) = aug8<T>(mk, one3);
+        if (tid < KB) *reinterpret_cast<v8 *>(dst + R::OFF_AK + tid * 16) = aug8<T>(mk, one3);
+    };
+
+    fetch(s_begin);
+    stash(0);
+    __syncthreads();
+    for (int s = s_begin; s < s_end; ++s) {
+        const bool dead = e.dead[b * p.S + s] != 0;
+        const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
+        const float bscale = dead ? 0.0f : kLog2e;   // a row with every key masked takes no bias
+        const unsigned char *buf = lds + ((s - s_begin) & 1) * R::LDS_BYTES;
         // the wave's operands of this row: Q scaled (with its rounding residue for small head
         // dims), dO, ones against the mask columns, -LSE and -delta against ones
         v8 qf[KS], gf[KS], qlo[KSD];
@@ -154,8 +162,7 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                 gf[ks] = aug8<T>(pack_split3<T>(-delta_n), zero3);
             }
         }
-        __syncthreads();
-        fetch(min(s + 1, s_end - 1));
+        fetch(min(s + 1, s_end - 1));   // in flight during the row's tiles
 
         if (active) {
 #pragma unroll
@@ -180,10 +187,10 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                         v8 ka = zero8<T>(), va = zero8<T>();
                         if (d0 < D) {
                             const int o = R::swz(kb + li, 2 * ks + g);
-                            ka = *reinterpret_cast<const v8 *>(lds + R::OFF_K + o);
-                            va = *reinterpret_cast<const v8 *>(lds + R::OFF_V + o);
+                            ka = *reinterpret_cast<const v8 *>(buf + R::OFF_K + o);
+                            va = *reinterpret_cast<const v8 *>(buf + R::OFF_V + o);
                         } else if (d0 == AUGC) {
-                            ka = *reinterpret_cast<const v8 *>(lds + R::OFF_AK + (kb + li) * 16);
+                            ka = *reinterpret_cast<const v8 *>(buf + R::OFF_AK + (kb + li) * 16);
                             va = vaug;
                         }
                         acc = Mfma<T>::mma(ka, qf[ks], acc);                                   // log2 P^T
@@ -200,6 +207,10 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        // the next row's keys into the other buffer (everybody left it at the barrier before this
+        // row); one barrier per row
+        stash(((s - s_begin) & 1) ^ 1);
+        __syncthreads();
     }
 
     // the partial of this chunk: lane = query li, registers 4rr .. 4rr+3 = keys 8rr + 4g ..
