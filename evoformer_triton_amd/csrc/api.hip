@@ -90,7 +90,9 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 }
 
 // Rows of more than 384 keys with a dBias to sum (up to there the dQ kernel that keeps the sums
-// has two query tiles per workgroup, beyond one): dQ from that same kernel, and the dBias
+// has two query tiles per workgroup, beyond one; with at most four (batch, head) pairs, where
+// that kernel fills the chip only with many chunks of S and so many partials, from 257 keys
+// on: S = N = 384, H = 4: backward 322 against 364 us, with H = 8 857 against 827 us): dQ from that same kernel, and the dBias
 // partials from a kernel of their own that forms dS a second time (dQ and partials, S = N:
 // N = 512: 436 against 483 us, N = 768: 1.32 against 1.67 ms, N = 1024, S = 256: 0.80 against
 // 1.56 ms; N = 384: 211 against 204 us, and with few S rows the second kernel's start-up shows;
@@ -98,7 +100,7 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 // against 661 us there, 0.65 against 1.38 ms and 740 against 793 us at N = 768).
 // Bit 0x2000 of flags (not part of the public interface) selects the one kernel, for comparison.
 static bool dq_split_ok(const EvoAttnParams &p) {
-    if (!p.dbias || p.S < 64 || p.N <= (p.D == 32 ? 384 : 512) || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
+    if (!p.dbias || p.S < 64 || p.N <= (p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384) || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.D <= 32 && p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs, in 32 registers
 }
 
