@@ -100,8 +100,11 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 // against 661 us there, 0.65 against 1.38 ms and 740 against 793 us at N = 768).
 // Bit 0x2000 of flags (not part of the public interface) selects the one kernel, for comparison.
 static bool dq_split_ok(const EvoAttnParams &p) {
-    if (!p.dbias || p.S < 64 || p.N <= (p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384) || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
-    return p.D <= 32 && p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs, in 32 registers
+    // shortest rows that go this way: where the kernel that keeps the sums has no form with
+    // prefetch (head dim 64 beyond 128 keys) or measured slower
+    const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
+    if (!p.dbias || p.S < 64 || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
+    return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }
 
 static bool dq_wide_ok(const EvoAttnParams &p) {
@@ -117,10 +120,11 @@ static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && p.S == 1
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t NT = (p.N + 31) / 32;
     if (dq_split_ok(p)) {
-        // the dBias kernel: one workgroup per block of 128 queries x 128 keys, (b, h) and chunk, two
+        // the dBias kernel: one workgroup per block of 128 queries x 128 keys (64 at head dim 64), (b, h) and chunk, two
         // workgroups per CU (256 CUs) at a time; among the chunk counts that give one to four rounds
         // the one that leaves the fewest slots idle in the last round (near ties: the fewest chunks)
-        const int64_t nb = (p.N + 127) / 128, base = nb * nb * p.B * p.H, slots = 512;
+        const int64_t kb = p.D == 64 ? 64 : 128;   // keys per block
+        const int64_t base = (int64_t)((p.N + 127) / 128) * ((p.N + kb - 1) / kb) * p.B * p.H, slots = 512;
         const int64_t lo = slots / base > 0 ? slots / base : 1, hi = (4 * slots + base - 1) / base;
         int64_t want = lo;
         double best = -1.0;

@@ -7,13 +7,14 @@
 // tiles per row that leaves a workgroup 32 queries for all the keys it stages (N = 768: dQ in
 // 1.67 ms against 0.68 ms without the sum).  For such rows dQ comes from the kernel that knows
 // nothing of dBias, and this kernel forms dS a second time: a workgroup of 4 waves owns a block
-// of 128 queries x 128 keys of one (b, h) for a chunk of S rows, a wave 32 queries x 4 key
-// tiles, whose running sums (64 registers) and bias tiles (32, as 16-bit pairs) stay resident.  Per S row the
-// workgroup stages its 128 keys (K with the mask columns, V) in LDS, the waves fetch their own
-// query rows (Q, dO, LSE, delta, as written by the dQ kernel); both are requested one row ahead
-// into registers, and the keys go to the other of two LDS buffers after the row's tiles: one
-// barrier per row.  Per tile: two score MFMA chains, exp2, a multiply and 16 additions; no
-// conversions, no gradient matmul.  One partial per chunk; `dbias_reduce` adds them in order.
+// of 128 queries x 128 keys (64 at head dim 64) of one (b, h) for a chunk of S rows, a wave 32
+// queries x 4 (2) key tiles, whose running sums (64 registers) and bias tiles (32, as 16-bit
+// pairs) stay resident.  Per S row the workgroup stages its keys (K with the mask columns, V)
+// in LDS, the waves fetch their own query rows (Q, dO, LSE, delta, as written by the dQ kernel);
+// both are requested one row ahead into registers, and the keys go to the other of two LDS
+// buffers after the row's tiles: one barrier per row.  Per tile: two score MFMA chains, exp2, a
+// multiply and 16 additions; no conversions, no gradient matmul.  One partial per chunk;
+// `dbias_reduce` adds them in order.
 #include "bwd_common.h"
 #include "kernels.h"
 
@@ -27,7 +28,9 @@ template <int D>
 struct DbGeo {
     static constexpr int C = D / 8;                          // 16-byte chunks per row
     static constexpr int RPB = 16 / C > 0 ? 16 / C : 1;      // rows per 256 bytes
-    static constexpr int KB = 128, QB = 128, TPW = 4;        // keys, queries per workgroup; key tiles per wave
+    // keys, queries per workgroup; key tiles per wave (head dim 64: half the keys, its operands
+    // take the registers of two tiles' sums and bias)
+    static constexpr int TPW = D <= 32 ? 4 : 2, KB = TPW * 32, QB = 128;
     static constexpr int OFF_K = 0, OFF_V = KB * D * 2, OFF_AK = 2 * KB * D * 2;
     static constexpr int LDS_BYTES = OFF_AK + KB * 16;
     static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
