@@ -102,8 +102,11 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 static bool dq_split_ok(const EvoAttnParams &p) {
     // shortest rows that go this way: where the kernel that keeps the sums has no form with
     // prefetch (head dim 64 beyond 128 keys) or measured slower
+    // fewest S rows: the second kernel's start-up has to pay (N = 768, D = 32: ahead from 8 rows on;
+    // N = 512: 72 against 66 us at 32 rows)
+    const int min_s = p.D == 32 && p.N > 512 ? 8 : 64;
     const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
-    if (!p.dbias || p.S < 64 || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
+    if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }
 

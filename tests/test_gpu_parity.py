@@ -384,11 +384,13 @@ def test_dq_where_no_dbias_is_asked_for(E, case):
 
 @pytest.mark.parametrize("case", [(1, 64, 416, 1, 32, "add", torch.bfloat16), (1, 70, 520, 2, 16, "bool", torch.bfloat16),
                                   (1, 64, 530, 1, 8, "soft", torch.float16), (2, 66, 400, 1, 32, "bool", torch.float16),
-                                  (1, 64, 200, 2, 64, "add", torch.bfloat16), (1, 65, 322, 1, 64, "bool", torch.float16)],
+                                  (1, 64, 200, 2, 64, "add", torch.bfloat16), (1, 65, 322, 1, 64, "bool", torch.float16),
+                                  (1, 9, 640, 2, 32, "add", torch.bfloat16)],
                          ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
 def test_long_rows_sum_dbias_in_a_kernel_of_its_own(E, case):
     """Rows of more than 384 keys (512 at head dims 8 and 16; 256 at head dim 32 with at most four
-    (batch, head) pairs; 128 at head dim 64) with at least 64 S rows: dQ from
+    (batch, head) pairs; 128 at head dim 64) with at least 64 S rows (8 beyond 512 keys at head
+    dim 32): dQ from
     the kernel whose waves own their query rows, the dBias partials from a second kernel that
     forms dS again (`evoattn_kernels` names both).  Against the CPU oracle in fp32, and against
     the one kernel that does both (flag bit 0x2000) to a 16-bit unit in the last place."""
