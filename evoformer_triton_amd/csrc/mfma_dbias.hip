@@ -175,10 +175,12 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                     f32x16 acc, dp;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
-                        unsigned w = bres[j][i];
-                        asm volatile("" : "+v"(w));   // unpack per use: expanded once and for all the tiles would take twice the registers
+                        // unpack per use: expanded once and for all the tiles would take twice the
+                        // registers (the empty statement "changes" the resident register in place, so
+                        // that its expansion cannot be moved out of the loop over S, at no copy)
+                        asm volatile("" : "+v"(bres[j][i]));
                         float lo, hi;
-                        unpack2<T>(w, lo, hi);
+                        unpack2<T>(bres[j][i], lo, hi);
                         acc[2 * i] = lo * bscale;
                         acc[2 * i + 1] = hi * bscale;
                     }

@@ -285,11 +285,12 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
                     for (int k = 0; k < 4; ++k) {
                         // (the pairs are unpacked per row: expanded once and for all they
                         // would take twice the registers)
-                        unsigned w0 = bres[4 * qt + k].x, w1 = bres[4 * qt + k].y;
-                        asm volatile("" : "+v"(w0), "+v"(w1));
+                        // (the empty statement "changes" the resident registers in place: their
+                        // expansion cannot be moved out of the loop over S, and no copy is made)
+                        asm volatile("" : "+v"(bres[4 * qt + k].x), "+v"(bres[4 * qt + k].y));
                         float f0, f1, f2, f3;
-                        unpack2<T>(w0, f0, f1);
-                        unpack2<T>(w1, f2, f3);
+                        unpack2<T>(bres[4 * qt + k].x, f0, f1);
+                        unpack2<T>(bres[4 * qt + k].y, f2, f3);
                         acc[4 * k] = f0 * bscale; acc[4 * k + 1] = f1 * bscale;
                         acc[4 * k + 2] = f2 * bscale; acc[4 * k + 3] = f3 * bscale;
                     }
