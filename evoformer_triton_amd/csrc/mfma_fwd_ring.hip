@@ -247,6 +247,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 if (2 * ks + g < C) scaled_hilo8<T>(qraw[ks], cq, qf[ks], qlo[ks]);
             }
             v8 qaug = aug8<T>(ones3<T>(), uint2{0u, 0u});   // ones x mask columns, -mf x ones
+            v8 qaug_hi0 = g ? zero8<T>() : qaug;             // the same as a whole k-step: zeros in the upper half
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -288,15 +289,14 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                             k1 = *reinterpret_cast<const v8 *>(buf + R::swz(kb + 32 + li, ch < C ? ch : 0));
                             qb = qf[ks];
                         }
-                    } else {  // the mask k-step: lane group 0
-                        k0 = zero8<T>();
-                        k1 = zero8<T>();
-                        qb = zero8<T>();
-                        if (g == 0) {
-                            k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
-                            k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
-                            qb = qaug;
-                        }
+                    } else {
+                        // the mask k-step: its columns sit in the lower half (lane group 0).  The
+                        // upper half of the Q side is zero, so the upper half of the K side may hold
+                        // any finite values: both lane groups read the same chunk (no registers to
+                        // clear, no exec mask to change per step)
+                        k0 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + li) * 16);
+                        k1 = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (kb + 32 + li) * 16);
+                        qb = qaug_hi0;
                     }
                     if (ks == 0 && BIASK == 1 && !dead) {  // uniform
                         a0 = Mfma<T>::mma(k0, qb, btile[2 * step]);
@@ -352,6 +352,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     // from the next scores on the MFMA subtracts m itself
                     mf = fabsf(m) <= 1024.0f ? m : 0.0f;
                     qaug = aug8<T>(ones3<T>(), pack_split3<T>(-mf));
+                    qaug_hi0 = g ? zero8<T>() : qaug;
                 }
             };
             // ---- part 2: P = exp2, rounded to T, and this lane's sum of the rounded values
