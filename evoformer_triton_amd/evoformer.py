@@ -19,7 +19,7 @@ Differences from the reference, all supersets:
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Sequence
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -123,7 +123,20 @@ def _check_qkv(Q, K, V):
         raise RuntimeError("EvoformerAttention runs on the GPU only (no CPU implementation); move Q, K, V to one cuda device")
 
 
-def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
+def _prep_bytes_upper(lib, p):
+    """Size of the prep buffer that holds for any alignment of the bias: with few S rows the
+    library reads an aligned bias in place and needs less; an odd address asks for the most."""
+    saved = p.bias
+    if saved is not None:
+        p.bias = ctypes.c_void_p(1)
+    n = lib.evoattn_prep_bytes(ctypes.byref(p))
+    p.bias = saved
+    return n
+
+
+def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
+    """Validate, allocate O / LSE / prep with torch and enqueue the forward on the current
+    stream.  Returns what the backward needs: the tensors as the kernels saw them."""
     _check_qkv(Q, K, V)
     lib = _lib.load()
     B, S, N, H, D = Q.shape
@@ -134,22 +147,38 @@ def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
         O = torch.empty_like(Qc)                               # evoformer.py:654
         lse = torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32)   # :669-671
         p = _params(Qc, Kc, Vc, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
-        prep = _alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), Q.device)
+        nbytes = _prep_bytes_upper(lib, p) if prep_upper else lib.evoattn_prep_bytes(ctypes.byref(p))
+        prep = _alloc_bytes(nbytes, Q.device)
         p.prep, p.prep_bytes = _ptr(prep), prep.numel()
         _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(Q.device)), "evoattn_fwd")
+    mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
+    bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+    return Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta
+
+
+def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
+    if torch.compiler.is_compiling():
+        # under torch.compile the device work is the registered operator (opaque to the tracer)
+        O, lse, prep = torch.ops.evoattn.fwd(Q, K, V, res_mask, pair_bias, layout == "ds4sci")
+        ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep)
+        ctx.layout, ctx.through_ops = layout, True
+        return O
+    Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta = _fwd_impl(Q, K, V, res_mask, pair_bias, layout)
     ctx.save_for_backward(Qc, Kc, Vc, mask, bias, O, lse, prep)  # :729
-    ctx.layout = layout
-    ctx.mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
-    ctx.bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+    ctx.layout, ctx.through_ops = layout, False
+    ctx.mask_meta, ctx.bias_meta = mask_meta, bias_meta
     return O
 
 
-def _backward(ctx, dO, need_dmask, need_dbias):
+def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_meta, need_dmask, need_dbias,
+              prep_valid=True):
+    """Allocate the gradients and the workspace and enqueue the backward; `mask` and `bias`
+    are the tensors the forward's kernels saw.  Returns (dQ, dK, dV, dmask, dbias) with the
+    last two in the shape and dtype of the caller's tensors, or None."""
     lib = _lib.load()
-    Q, K, V, mask, bias, O, lse, prep = ctx.saved_tensors
     B, S, N, H, D = Q.shape
-    mask_kind, mstr, mask_orig = ctx.mask_meta
-    bias_dt, bstr, bias_orig = ctx.bias_meta
+    mask_kind, mstr, mask_orig = mask_meta
+    bias_dt, bstr, bias_orig = bias_meta
     dO = dO.contiguous()                                        # the reference asserts this, :747
     if dO.dtype != Q.dtype:
         dO = dO.to(Q.dtype)
@@ -157,7 +186,7 @@ def _backward(ctx, dO, need_dmask, need_dbias):
     want_dmask = bool(need_dmask and mask is not None and mask.is_floating_point())
     with torch.cuda.device(Q.device):
         dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)   # :749-751
-        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, ctx.layout)
+        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
         p.dout, p.dq, p.dk, p.dv = _ptr(dO), _ptr(dQ), _ptr(dK), _ptr(dV)
         dbias = dmask = None
         if want_dbias:
@@ -169,8 +198,11 @@ def _backward(ctx, dO, need_dmask, need_dbias):
             p.dmask = _ptr(dmask)
         ws = _alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), Q.device)
         p.workspace, p.workspace_bytes = _ptr(ws), ws.numel()
+        if not prep_valid:                                       # not the forward's tensors: prepare again
+            prep = _alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), Q.device)
         p.prep, p.prep_bytes = _ptr(prep), prep.numel()
-        p.flags |= _lib.EVO_FLAG_PREP_VALID                      # same bias and mask as the forward
+        if prep_valid:
+            p.flags |= _lib.EVO_FLAG_PREP_VALID                  # same bias and mask as the forward
         _lib.check(lib.evoattn_bwd(ctypes.byref(p), _stream(Q.device)), "evoattn_bwd")
     if dbias is not None:
         shape, dtype = bias_orig
@@ -187,6 +219,102 @@ def _backward(ctx, dO, need_dmask, need_dbias):
             dmask = dmask.sum(1, keepdim=True)
         dmask = dmask.to(dtype)
     return dQ, dK, dV, dmask, dbias
+
+
+def _backward(ctx, dO, need_dmask, need_dbias):
+    if ctx.through_ops:
+        Q, K, V, res_mask, pair_bias, O, lse, prep = ctx.saved_tensors
+        dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep,
+                                                         ctx.layout == "ds4sci", bool(need_dbias), bool(need_dmask))
+        want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
+        return dQ, dK, dV, (dmask if want_dmask else None), (dbias if need_dbias and pair_bias is not None else None)
+    Q, K, V, mask, bias, O, lse, prep = ctx.saved_tensors
+    return _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, ctx.layout, ctx.mask_meta, ctx.bias_meta,
+                     need_dmask, need_dbias)
+
+
+# ---- the same two calls as registered operators (torch.ops.evoattn.fwd / .bwd) ------------------
+# Opaque to torch.compile's tracer, with shape-only implementations for it and an autograd
+# formula, so that a model that calls EvoformerAttention.apply compiles without a graph break.
+
+@torch.library.custom_op("evoattn::fwd", mutates_args=(), device_types="cuda")
+def _op_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
+            pair_bias: Optional[torch.Tensor], per_head: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(O, LSE [B,H,S,N] fp32, prep bytes): the forward of EvoformerAttention (per_head False:
+    the reference's flat-reshape heads) or of DS4Sci_EvoformerAttention (per_head True)."""
+    out = _fwd_impl(Q, K, V, res_mask, pair_bias, "ds4sci" if per_head else "reference", prep_upper=True)
+    return out[5], out[6], out[7]
+
+
+@_op_fwd.register_fake
+def _(Q, K, V, res_mask, pair_bias, per_head):
+    B, S, N, H, D = Q.shape
+    lib = _lib.load()
+    p = EvoAttnParams()
+    p.B, p.S, p.N, p.H, p.D = B, S, N, H, D
+    p.dtype = _DTYPES[Q.dtype]
+    p.bias_dtype, p.mask_kind = _lib.EVO_NONE, _lib.EVO_MASK_NONE
+    if pair_bias is not None:
+        p.bias = ctypes.c_void_p(1)
+        p.bias_dtype = _DTYPES[pair_bias.dtype if pair_bias.dtype in (torch.float32, Q.dtype) else torch.float32]
+        p.bias_stride_b = 0 if pair_bias.shape[0] == 1 else H * N * N
+        p.bias_stride_h, p.bias_stride_row = N * N, N
+    if res_mask is not None:
+        p.mask = ctypes.c_void_p(1)
+        p.mask_kind = _lib.EVO_MASK_BOOL if not res_mask.is_floating_point() else _MASK_KINDS.get(res_mask.dtype, _lib.EVO_MASK_F32)
+    nbytes = max(int(lib.evoattn_prep_bytes(ctypes.byref(p))), 256)
+    return (Q.new_empty(Q.shape), Q.new_empty((B, H, S, N), dtype=torch.float32),
+            Q.new_empty((nbytes,), dtype=torch.uint8))
+
+
+@torch.library.custom_op("evoattn::bwd", mutates_args=(), device_types="cuda")
+def _op_bwd(dO: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
+            pair_bias: Optional[torch.Tensor], O: torch.Tensor, lse: torch.Tensor, prep: torch.Tensor,
+            per_head: bool, need_dbias: bool, need_dmask: bool
+            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dQ, dK, dV, dMask, dBias) from the forward's inputs and outputs; a gradient that was not
+    asked for (or has no tensor to belong to) comes back as an empty tensor."""
+    B, S, N, H, D = Q.shape
+    Qc, Kc, Vc = Q.contiguous(), K.contiguous(), V.contiguous()
+    mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
+    bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
+    mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
+    bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+    # the prepared tiles are the forward's only if the kernels read the very same tensors
+    same = mask is res_mask and bias is pair_bias
+    dQ, dK, dV, dmask, dbias = _bwd_impl(dO, Qc, Kc, Vc, mask, bias, O.contiguous(), lse, prep,
+                                         "ds4sci" if per_head else "reference", mask_meta, bias_meta,
+                                         need_dmask, need_dbias, prep_valid=same)
+    none = Q.new_empty((0,))
+    return dQ, dK, dV, (none if dmask is None else dmask), (none.clone() if dbias is None else dbias)
+
+
+@_op_bwd.register_fake
+def _(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, per_head, need_dbias, need_dmask):
+    want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
+    want_dbias = need_dbias and pair_bias is not None
+    return (Q.new_empty(Q.shape), Q.new_empty(Q.shape), Q.new_empty(Q.shape),
+            res_mask.new_empty(res_mask.shape) if want_dmask else Q.new_empty((0,)),
+            pair_bias.new_empty(pair_bias.shape) if want_dbias else Q.new_empty((0,)))
+
+
+def _op_setup_context(ctx, inputs, output):
+    Q, K, V, res_mask, pair_bias, per_head = inputs
+    O, lse, prep = output
+    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep)
+    ctx.per_head = per_head
+
+
+def _op_backward(ctx, dO, dlse, dprep):
+    Q, K, V, res_mask, pair_bias, O, lse, prep = ctx.saved_tensors
+    need_dmask = bool(ctx.needs_input_grad[3] and res_mask is not None and res_mask.is_floating_point())
+    need_dbias = bool(ctx.needs_input_grad[4] and pair_bias is not None)
+    dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep,
+                                                     ctx.per_head, need_dbias, need_dmask)
+    return dQ, dK, dV, (dmask if need_dmask else None), (dbias if need_dbias else None), None
+
+
+_op_fwd.register_autograd(_op_backward, setup_context=_op_setup_context)
 
 
 class EvoformerAttention(torch.autograd.Function):

@@ -616,6 +616,84 @@ def test_checkpoint_recompute_and_no_grad(E):
     assert torch.equal(o2, plain["O"])
 
 
+OP_CASES = [  # (B, S, N, H, D, mask, bias dtype, per_head)
+    (1, 6, 256, 2, 32, "add", "q", False), (2, 3, 100, 2, 16, "bool", torch.float32, False),
+    (1, 4, 64, 4, 32, "soft", "q", True), (1, 2, 96, 2, 64, None, None, False),
+]
+
+
+@pytest.mark.parametrize("case", OP_CASES, ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_registered_operators_match_the_function(E, case):
+    """torch.ops.evoattn.fwd with its autograd formula gives bit for bit what the Function gives."""
+    B, S, N, H, D, mask, bias_dt, per_head = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, torch.bfloat16)
+    layout = "ds4sci" if per_head else "reference"
+    fmask = m is not None and m.dtype != torch.bool
+    plain = run_hip(E, Q, K, V, m, bias, dO, layout=layout, mask_grad=fmask)
+    dev = "cuda"
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, K, V))
+    b = None if bias is None else bias.to(dev).requires_grad_()
+    mm = None if m is None else m.to(dev)
+    if fmask:
+        mm.requires_grad_()
+    o, lse, _ = torch.ops.evoattn.fwd(q, k, v, mm, b, per_head)
+    o.backward(dO.to(dev))
+    torch.cuda.synchronize()
+    assert lse.shape == (B, H, S, N) and lse.dtype == torch.float32
+    assert torch.equal(o, plain["O"])
+    assert torch.equal(q.grad, plain["dQ"]) and torch.equal(k.grad, plain["dK"]) and torch.equal(v.grad, plain["dV"])
+    if b is not None:
+        assert b.grad.shape == bias.shape and torch.equal(b.grad, plain["dBias"])
+    if fmask:
+        assert torch.equal(mm.grad, plain["dMask"])
+
+
+def test_registered_operators_pass_opcheck(E):
+    """Schema, shape-only implementation and autograd registration, as torch.library checks them."""
+    Q, K, V, m, bias, dO = make_case(1, 3, 64, 2, 32, "bool", "q", torch.bfloat16)
+    dev = "cuda"
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, K, V))
+    b = bias.to(dev).requires_grad_()
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    torch.library.opcheck(torch.ops.evoattn.fwd, (q, k, v, m.to(dev), b, False), test_utils=tests)
+    with torch.no_grad():
+        o, lse, prep = torch.ops.evoattn.fwd(q, k, v, m.to(dev), b, False)
+    torch.library.opcheck(torch.ops.evoattn.bwd, (dO.to(dev), q.detach(), k.detach(), v.detach(), m.to(dev), b.detach(),
+                                                  o, lse, prep, False, True, False), test_utils=tests[:2])
+
+
+@pytest.mark.parametrize("case", [(1, 6, 256, 2, 32, "add", "q"), (2, 3, 100, 2, 16, "bool", torch.float32)],
+                         ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_torch_compile_traces_the_function_without_a_graph_break(E, case):
+    """A module that calls EvoformerAttention.apply between ordinary torch operations compiles as
+    one graph (fullgraph=True; the aot_eager backend: tracing, functionalisation and the
+    partitioned backward, no code generation) and returns what the eager module returns."""
+    B, S, N, H, D, mask, bias_dt = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, torch.bfloat16)
+    dev = "cuda"
+
+    def block(q, k, v, mask, bias, gate):
+        o = E.EvoformerAttention.apply(q, k, v, mask, bias * 1.0)
+        return torch.sigmoid(gate) * o
+
+    def run(fn):
+        q, k, v, g = (t.to(dev).requires_grad_() for t in (Q, K, V, dO))
+        b = bias.to(dev).requires_grad_()
+        out = fn(q, k, v, m.to(dev), b, g)
+        out.backward(dO.to(dev))
+        torch.cuda.synchronize()
+        return [out.detach(), q.grad, k.grad, v.grad, b.grad, g.grad]
+
+    want = run(block)
+    torch._dynamo.reset()
+    compiled = torch.compile(block, backend="aot_eager", fullgraph=True)
+    for _ in range(2):          # the second call replays the compiled graph
+        got = run(compiled)
+        for a, w in zip(got, want):
+            assert a.shape == w.shape and a.dtype == w.dtype
+            assert max_err(a, w) <= 1e-6 + 2.0 ** -7 * w.float().abs().max().item()
+
+
 def test_ds4sci_entry_point(E):
     Q, K, V, m, bias, dO = make_case(1, 3, 64, 4, 16, "soft", "q", torch.bfloat16)
     ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, layout="ds4sci", compute_dtype=torch.float32)
