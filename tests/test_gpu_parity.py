@@ -735,6 +735,61 @@ def test_reference_test_matrix(E, shape):
         assert torch.allclose(b, a, atol=1e-2, rtol=1e-2), f"{n}: max-abs {(a - b).abs().max().item():.3e}"   # test.py:73-80
 
 
+# ------------------------------------------------------------------ seeded sweep over the dispatch boundaries
+
+def _sweep_cases(n=64, seed=2024):
+    """Shapes drawn around the row lengths, S counts and head dims at which the library changes
+    kernels (128 / 256 / 384 / 512 / 768 keys; 1, 4, 8, 64 S rows; D = 8..64; bias dtype and
+    alignment; mask kind; layout; whether dBias is asked for)."""
+    import random
+    r = random.Random(seed)
+    edges = [31, 32, 33, 96, 127, 128, 129, 136, 200, 248, 255, 256, 257, 264, 320, 383, 384, 385, 392, 500, 511, 512,
+             513, 520, 640, 767, 768, 769, 1000]
+    cases = []
+    while len(cases) < n:
+        N, D = r.choice(edges), r.choice([8, 16, 32, 32, 64])
+        S = r.choice([1, 2, 4, 5, 8, 9, 33, 64, 65, 70])
+        B, H = r.choice([1, 1, 2]), r.choice([1, 2, 3, 4])
+        if B * H * S * N * N > 3.0e7:
+            continue
+        dt = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        mask = r.choice(["add", "bool", "soft", None])
+        if dt == torch.float16 and mask == "add":
+            mask = "bool"                       # -1e9 is not an fp16 value
+        bias_dt = r.choice(["q", "q", torch.float32, None])
+        cases.append((B, S, N, H, D, mask, bias_dt, r.choice(["reference", "ds4sci"]), dt, r.random() < 0.75,
+                      r.random() < 0.3, len(cases)))
+    return cases
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_seeded_sweep_over_dispatch_boundaries(E, case):
+    B, S, N, H, D, mask, bias_dt, layout, dt, bias_grad, dead_row, idx = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, dt, seed=500 + idx, std=0.7)
+    if dead_row and m is not None and mask != "soft":      # one S row with every key masked
+        m[0, S // 2] = False if m.dtype == torch.bool else -1e9
+    dev = "cuda"
+    on = lambda t: None if t is None else t.to(dev)
+    ref = eager.attention_fwd_bwd(on(Q), on(K), on(V), on(m), on(bias), on(dO), layout=layout,
+                                  compute_dtype=torch.float32, s_chunk=16)
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, K, V))
+    b = on(bias)
+    if b is not None and bias_grad:
+        b.requires_grad_()
+    o = E.evoformer_attention(q, k, v, on(m), b, layout=layout)
+    o.backward(on(dO))
+    torch.cuda.synchronize()
+    got = {"O": o.detach(), "dQ": q.grad, "dK": k.grad, "dV": v.grad}
+    names = ["O", "dQ", "dK", "dV"]
+    if b is not None and bias_grad:
+        got["dBias"] = b.grad
+        names.append("dBias")
+    for n in names:
+        assert torch.isfinite(got[n].float()).all(), f"{case}: {n} not finite"
+    # tolerance plus one ulp of the 16-bit result (2^-7 relative covers bf16; fp16 is finer)
+    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+
+
 # ------------------------------------------------------------------ full-size benchmark configurations
 
 @pytest.mark.parametrize("cfg", ["C2", "C3", "C4", "C5"])
