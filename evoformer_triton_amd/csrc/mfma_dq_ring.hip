@@ -352,10 +352,6 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         gf[ks] = aug8<T>(pack_split3<T>(-dl), zero3);    // -delta x ones
                     }
                 }
-                if (kill) {  // no gradient through the scores of such a row: dP - delta := 0
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) gf[ks] = zero8<T>();
-                }
             }
 
             if (MID) fetch_part(t + 1, SPLIT, IPW);
@@ -367,7 +363,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     const int tb = jj * KQ + kq;         // tile inside the stage
                     const int kt = blk * TPB + tb;
                     if (MID && jj == TPW - 1) stash_part(t + 1, 0, SPLIT);
-                    if (qact && kt < NT) {  // wave-uniform
+                    // wave-uniform; no gradient goes through the scores of a row that a bool mask drops
+                    // entirely: its tiles are skipped, dQ stays zero and dBias unchanged
+                    if (qact && kt < NT && !kill) {
                         const int slot = blk * TPW + jj;
                         v8 ka[KS], va[KS];
 #pragma unroll
@@ -379,7 +377,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                                 const int o = R::swz(tb * 32 + li, 2 * ks + g);
                                 ka[ks] = *reinterpret_cast<const v8 *>(buf + o);
                                 va[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_V + o);
-                            } else if (d0 == AUGC) {
+                            } else if (d0 == AUGC || (D >= 16 && ks == KS - 1)) {
+                                // The extra columns.  From head dim 16 on they have a k-step of their own, whose
+                                // upper half (lane group 1) is zero on the query side: there the key side may hold
+                                // any finite values, so both lane groups read the same columns and no lane is
+                                // cleared or masked per tile.
                                 ka[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (tb * 32 + li) * 16);  // mask x ones, ones x -lse
                                 va[ks] = aug8<T>(one3, zero3);                                                 // ones x -delta
                             }
@@ -398,8 +400,6 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                             if (G::RESID && ks < KSD) acc = Mfma<T>::mma(ka[ks], qlo[ks], acc);
                             dp = Mfma<T>::mma(va[ks], gf[ks], dp);     // dP^T - delta
                         }
-                        // (in a row that a bool mask drops entirely dO and -delta were zeroed
-                        // above, so dP - delta and with it dS are zero)
                         float ds[16];
 #pragma unroll
                         for (int r = 0; r < 16; ++r) ds[r] = fast_exp2(acc[r]) * dp[r];
