@@ -45,6 +45,11 @@ def _units():
         units.append((f"mfma_kvr_d{d}", "mfma_dkdv_ring.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_dqw_d{d}", "mfma_dq_wide.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_dbias_d{d}", "mfma_dbias.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
+    # head dim 128: the one-workgroup-per-problem kernels (the chunk-of-rows kernels and the
+    # dBias kernel keep more per wave than 256 registers hold at that width)
+    units.append(("mfma_fwd_d128", "mfma_fwd.hip", ["-DEVO_D=128", *VGPR_FORM]))
+    units.append(("mfma_bwd_d128", "mfma_bwd.hip", ["-DEVO_D=128", *VGPR_FORM]))
+    units.append(("mfma_dqw_d128", "mfma_dq_wide.hip", ["-DEVO_D=128", *VGPR_FORM]))
     return units
 
 

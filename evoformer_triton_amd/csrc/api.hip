@@ -43,7 +43,7 @@ static int check_common(const EvoAttnParams *p) {
 static bool mfma_ok(const EvoAttnParams &p, int pass) {
     if (p.flags & EVO_FLAG_FORCE_GENERIC) return false;
     if (p.dtype != EVO_BF16 && p.dtype != EVO_F16) return false;
-    if (p.D != 8 && p.D != 16 && p.D != 32 && p.D != 64) return false;
+    if (p.D != 8 && p.D != 16 && p.D != 32 && p.D != 64 && p.D != 128) return false;
     if (p.stride_b % 8 || p.stride_h % 8 || p.stride_s % 8 || p.stride_n % 8) return false;
     if (!aligned(p.q, 16) || !aligned(p.k, 16) || !aligned(p.v, 16) || !aligned(p.o, 16)) return false;
     if (pass == EVO_PASS_BWD) {
@@ -106,6 +106,7 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     // N = 512: 72 against 66 us at 32 rows)
     const int min_s = p.D == 32 && p.N > 512 ? 8 : 64;
     const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
+    if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }

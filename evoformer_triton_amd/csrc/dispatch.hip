@@ -21,6 +21,16 @@ EVO_DECL(16)
 EVO_DECL(32)
 EVO_DECL(64)
 #undef EVO_DECL
+// head dim 128: the one-workgroup-per-problem kernels only
+int launch_mfma_fwd_d128(const EvoAttnParams &, const Extra &, hipStream_t);
+int launch_mfma_dq_d128(const EvoAttnParams &, const Extra &, hipStream_t);
+int launch_mfma_dkdv_d128(const EvoAttnParams &, const Extra &, hipStream_t);
+int launch_mfma_dqw_d128(const EvoAttnParams &, const Extra &, hipStream_t);
+static int unbuilt(const EvoAttnParams &, const Extra &, hipStream_t) { return EVO_EUNSUPPORTED; }
+#define launch_mfma_fwdr_d128 unbuilt
+#define launch_mfma_dqr_d128 unbuilt
+#define launch_mfma_kvr_d128 unbuilt
+#define launch_mfma_dbias_d128 unbuilt
 
 #define EVO_ROUTE(name)                                                       \
     int launch_mfma_##name(const EvoAttnParams &p, const Extra &e, hipStream_t st) { \
@@ -29,6 +39,7 @@ EVO_DECL(64)
             case 16: return launch_mfma_##name##_d16(p, e, st);               \
             case 32: return launch_mfma_##name##_d32(p, e, st);               \
             case 64: return launch_mfma_##name##_d64(p, e, st);               \
+            case 128: return launch_mfma_##name##_d128(p, e, st);             \
         }                                                                     \
         return EVO_EUNSUPPORTED;                                              \
     }

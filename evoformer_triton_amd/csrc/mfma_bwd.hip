@@ -340,7 +340,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 #endif
 
 template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
-__global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
+__global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef KvGeo<D> R;
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
@@ -631,20 +631,26 @@ static int dq_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.bias_dtype == EVO_NONE ? dq_ntw<T, D, false>(p, e, st) : dq_ntw<T, D, true>(p, e, st);
 }
 
+template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
+static int dkdv_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    const unsigned grid = (unsigned)((p.N + NW * 32 - 1) / (NW * 32)) * (unsigned)(p.B * p.H * p.S);
+    constexpr int lds = KvGeo<D>::lds_bytes(ROWS);   // at most 56 KB up to head dim 64, 100 KB at 128
+    auto kern = mfma_dkdv<T, D, HAS_BIAS, NW, ROWS>;
+    if constexpr (lds > 64 * 1024) {
+        static PerDevice done{};
+        if (const int rc = ensure_dynamic_lds((const void *)kern, lds, done, nullptr)) return rc;
+    }
+    kern<<<grid, NW * 64, lds, st>>>(p, e);
+    return hip_rc();
+}
+
 template <typename T, int D, int NW>
 static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const unsigned grid = (unsigned)((p.N + NW * 32 - 1) / (NW * 32)) * (unsigned)(p.B * p.H * p.S);
     typedef KvGeo<D> R;
-    if (NW == 4 && p.N <= 128) {
-        constexpr int lds = R::lds_bytes(128);
-        if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW, 128><<<grid, NW * 64, lds, st>>>(p, e);
-        else mfma_dkdv<T, D, true, NW, 128><<<grid, NW * 64, lds, st>>>(p, e);
-    } else {
-        constexpr int lds = R::lds_bytes(R::BQS);   // at most 56 KB
-        if (p.bias_dtype == EVO_NONE) mfma_dkdv<T, D, false, NW, R::BQS><<<grid, NW * 64, lds, st>>>(p, e);
-        else mfma_dkdv<T, D, true, NW, R::BQS><<<grid, NW * 64, lds, st>>>(p, e);
-    }
-    return hip_rc();
+    if (NW == 4 && p.N <= 128)
+        return p.bias_dtype == EVO_NONE ? dkdv_launch<T, D, false, NW, 128>(p, e, st) : dkdv_launch<T, D, true, NW, 128>(p, e, st);
+    return p.bias_dtype == EVO_NONE ? dkdv_launch<T, D, false, NW, R::BQS>(p, e, st)
+                                    : dkdv_launch<T, D, true, NW, R::BQS>(p, e, st);
 }
 
 // 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys: measured faster

@@ -39,7 +39,7 @@ struct DqWideGeo {
 typedef short s16x4w __attribute__((ext_vector_type(4)));
 
 template <typename T, int D, bool HAS_BIAS, int NW, bool WRITE_DS>
-__global__ void __launch_bounds__(NW * 64, NW == 8 ? (D <= 32 ? 4 : 2) : 3) mfma_dq_wide(EvoAttnParams p, Extra e) {
+__global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4 : 2) : 3) mfma_dq_wide(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef DqWideGeo<D> R;
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;

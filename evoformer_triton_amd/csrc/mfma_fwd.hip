@@ -28,7 +28,7 @@
 namespace evo {
 
 template <typename T, int D, bool HAS_BIAS, int NW>
-__global__ void __launch_bounds__(NW * 64, D == 64 ? 2 : NW == 8 ? 4 : 3) mfma_fwd(EvoAttnParams p, Extra e) {
+__global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_fwd(EvoAttnParams p, Extra e) {
     constexpr int NTH = NW * 64;                  // threads per workgroup
     constexpr int BQ = NW * 32;                   // query rows per workgroup
     constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round

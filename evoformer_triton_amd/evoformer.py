@@ -10,7 +10,7 @@ Differences from the reference, all supersets:
   * `res_mask` may be None, a bool keep-mask (the reference's convention, evoformer.py:69)
     or an additive floating mask (the DS4Sci convention, speed_benchmark.py:24,84);
   * `pair_bias` may be None (the reference crashes on None, evoformer.py:651-652);
-  * head dims 8 and 16 and any N are accepted; fp32 inputs run an all-fp32 check mode;
+  * head dims 8, 16 and 128 and any N are accepted; fp32 inputs run an all-fp32 check mode;
   * dBias comes from a deterministic two-stage sum, not float atomics (evoformer.py:458),
     and is returned in the bias's own dtype;
   * a floating mask that requires grad receives its gradient (the reference returns None,

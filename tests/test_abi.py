@@ -110,7 +110,10 @@ def test_path_selection(lib):
     p = good(dtype=_lib.EVO_F32)
     assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"            # check mode
     p = good(D=128)
-    assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"
+    assert lib.evoattn_path(ctypes.byref(p), 0) == b"mfma" and lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
+    assert b"ring" not in lib.evoattn_kernels(ctypes.byref(p), 0) + lib.evoattn_kernels(ctypes.byref(p), 1)
+    p = good(D=24)
+    assert lib.evoattn_check(ctypes.byref(p), 0) == _lib.EVO_EUNSUPPORTED
     p = good()
     p.flags = _lib.EVO_FLAG_FORCE_GENERIC
     assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"

@@ -488,11 +488,56 @@ def test_fp32_check_mode_small_dims_and_ragged(E):
         assert_close(got, ref, F32_TOL, what=f"fp32 {B,S,N,H,D}")
 
 
+D128_CASES = [  # B, S, N, H, mask, bias dtype, layout, dtype, dBias asked for
+    (1, 2, 48, 2, "add", "q", "reference", torch.bfloat16, True),
+    (1, 3, 128, 2, "bool", torch.float32, "reference", torch.bfloat16, True),
+    (2, 5, 200, 2, "soft", "q", "ds4sci", torch.bfloat16, True),
+    (1, 4, 256, 2, "add", "q", "reference", torch.bfloat16, True),
+    (1, 70, 257, 1, "bool", "q", "reference", torch.float16, True),      # enough S rows for the other dims' dBias kernel
+    (1, 2, 520, 1, None, None, "reference", torch.bfloat16, False),
+    (4, 1, 384, 4, "bool", torch.float32, "reference", torch.bfloat16, True),   # S = 1: dBias written by the dQ kernel
+    (2, 1, 300, 2, "add", "q", "ds4sci", torch.bfloat16, True),
+    (1, 9, 640, 1, "add", "q", "reference", torch.bfloat16, False),      # bias as a constant
+    (1, 1, 1100, 1, "bool", "q", "reference", torch.bfloat16, True),
+]
+
+
+@pytest.mark.parametrize("case", D128_CASES, ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_head_dim_128_on_the_matrix_core(E, case):
+    """Head dim 128 runs the one-workgroup-per-problem matrix-core kernels (`evoattn_path`
+    says so through the C ABI) and meets the same bound against the fp32 eager oracle."""
+    from evoformer_triton_amd import _lib
+    B, S, N, H, mask, bias_dt, layout, dt, bias_grad = case
+    D = 128
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, dt, seed=77, std=0.7)
+    dev = "cuda"
+    on = lambda t: None if t is None else t.to(dev)
+    ref = eager.attention_fwd_bwd(on(Q), on(K), on(V), on(m), on(bias), on(dO), layout=layout,
+                                  compute_dtype=torch.float32, s_chunk=16)
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, K, V))
+    b = on(bias)
+    if b is not None and bias_grad:
+        b.requires_grad_()
+    o = E.evoformer_attention(q, k, v, on(m), b, layout=layout)
+    o.backward(on(dO))
+    torch.cuda.synchronize()
+    got = {"O": o.detach(), "dQ": q.grad, "dK": k.grad, "dV": v.grad}
+    names = ["O", "dQ", "dK", "dV"]
+    if b is not None and bias_grad:
+        got["dBias"] = b.grad
+        names.append("dBias")
+    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+    lib = _lib.load()
+    lse = torch.empty((B, H, S, N), device=dev)
+    mm, mk, mstr = E._prep_mask(on(m), B, S, N, q.device)
+    bb, bdt, bstr = E._prep_bias(b, B, H, N, q.dtype, q.device)
+    p = E._params(q.detach(), k.detach(), v.detach(), mm, mk, mstr, bb, bdt, bstr, torch.empty_like(q), lse, layout)
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_FWD) == b"mfma"
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_BWD) == b"mfma"
+
+
 def test_generic_fallbacks(E):
-    """Head dim 128 and a 2-byte-aligned storage offset are served by the plain kernels."""
-    Q, K, V, m, bias, dO = make_case(1, 2, 48, 2, 128, "add", "q", torch.bfloat16)
-    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
-    assert_close(run_hip(E, Q, K, V, m, bias, dO), ref, BF16_TOL, what="D=128")
+    """A 2-byte-aligned storage offset is served by the plain kernels."""
     Q, K, V, m, bias, dO = make_case(1, 2, 48, 2, 32, "add", "q", torch.bfloat16)
     ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
     dev = "cuda"
