@@ -10,7 +10,8 @@ Differences from the reference, all supersets:
   * `res_mask` may be None, a bool keep-mask (the reference's convention, evoformer.py:69)
     or an additive floating mask (the DS4Sci convention, speed_benchmark.py:24,84);
   * `pair_bias` may be None (the reference crashes on None, evoformer.py:651-652);
-  * head dims 8, 16 and 128 and any N are accepted; fp32 inputs run an all-fp32 check mode;
+  * every head dim up to 128 and any N are accepted (8, 16, 32, 64, 128 as they are, the others
+    padded with zero columns to the next of these); fp32 inputs run an all-fp32 check mode;
   * dBias comes from a deterministic two-stage sum, not float atomics (evoformer.py:458),
     and is returned in the bias's own dtype;
   * a floating mask that requires grad receives its gradient (the reference returns None,
@@ -83,7 +84,7 @@ def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
-def _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout):
+def _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=None):
     B, S, N, H, D = Q.shape
     p = EvoAttnParams()
     p.B, p.S, p.N, p.H, p.D = B, S, N, H, D
@@ -92,7 +93,7 @@ def _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
     p.mask_kind = mask_kind
     p.dbias_dtype = _lib.EVO_F32
     p.flags = FLAGS
-    p.scale = float(D) ** -0.5          # evoformer.py:646
+    p.scale = float(head_dim or D) ** -0.5          # evoformer.py:646 (the caller's D where the tensors are padded)
     p.stride_b, p.stride_h, p.stride_s, p.stride_n = _q_strides(B, S, N, H, D, layout)
     p.bias_stride_b, p.bias_stride_h, p.bias_stride_row = bstr
     p.mask_stride_b, p.mask_stride_s = mstr
@@ -100,6 +101,23 @@ def _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
     p.bias, p.mask = _ptr(bias), _ptr(mask)
     p.o, p.lse = _ptr(O), _ptr(lse)
     return p
+
+
+_HEAD_DIMS = (8, 16, 32, 64, 128)     # what the library is built for
+
+
+def _pad_head_dim(D):
+    """The head dim the kernels run a caller's D at: the next one the library is built for.
+    Zero columns change neither Q K^T nor the first D columns of P V; the softmax scale stays
+    the caller's D^-0.5."""
+    for d in _HEAD_DIMS:
+        if D <= d:
+            return d
+    raise ValueError(f"head dim {D} is beyond {_HEAD_DIMS[-1]}, the largest the kernels are built for")
+
+
+def _padded(t, Dp):
+    return t if t.shape[-1] == Dp else torch.nn.functional.pad(t, (0, Dp - t.shape[-1]))
 
 
 def _alloc_bytes(nbytes, device):
@@ -140,17 +158,21 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
     _check_qkv(Q, K, V)
     lib = _lib.load()
     B, S, N, H, D = Q.shape
+    Dp = _pad_head_dim(D)
     Qc, Kc, Vc = Q.contiguous(), K.contiguous(), V.contiguous()
+    Qp, Kp, Vp = _padded(Qc, Dp), _padded(Kc, Dp), _padded(Vc, Dp)
     mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
     bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
     with torch.cuda.device(Q.device):
-        O = torch.empty_like(Qc)                               # evoformer.py:654
+        O = torch.empty_like(Qp)                               # evoformer.py:654
         lse = torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32)   # :669-671
-        p = _params(Qc, Kc, Vc, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
+        p = _params(Qp, Kp, Vp, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
         nbytes = _prep_bytes_upper(lib, p) if prep_upper else lib.evoattn_prep_bytes(ctypes.byref(p))
         prep = _alloc_bytes(nbytes, Q.device)
         p.prep, p.prep_bytes = _ptr(prep), prep.numel()
         _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(Q.device)), "evoattn_fwd")
+        if Dp != D:
+            O = O[..., :D].contiguous()
     mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
     return Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta
@@ -182,11 +204,14 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
     dO = dO.contiguous()                                        # the reference asserts this, :747
     if dO.dtype != Q.dtype:
         dO = dO.to(Q.dtype)
+    Dp = _pad_head_dim(D)
+    if Dp != D:                                                  # zero columns, as in the forward
+        Q, K, V, O, dO = (_padded(t, Dp) for t in (Q, K, V, O, dO))
     want_dbias = bool(need_dbias and bias is not None)
     want_dmask = bool(need_dmask and mask is not None and mask.is_floating_point())
     with torch.cuda.device(Q.device):
         dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)   # :749-751
-        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout)
+        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
         p.dout, p.dq, p.dk, p.dv = _ptr(dO), _ptr(dQ), _ptr(dK), _ptr(dV)
         dbias = dmask = None
         if want_dbias:
@@ -204,6 +229,8 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
         if prep_valid:
             p.flags |= _lib.EVO_FLAG_PREP_VALID                  # same bias and mask as the forward
         _lib.check(lib.evoattn_bwd(ctypes.byref(p), _stream(Q.device)), "evoattn_bwd")
+    if Dp != D:
+        dQ, dK, dV = (t[..., :D].contiguous() for t in (dQ, dK, dV))
     if dbias is not None:
         shape, dtype = bias_orig
         dbias = dbias.reshape(B, 1, H, N, N)                    # :860
@@ -251,7 +278,7 @@ def _(Q, K, V, res_mask, pair_bias, per_head):
     B, S, N, H, D = Q.shape
     lib = _lib.load()
     p = EvoAttnParams()
-    p.B, p.S, p.N, p.H, p.D = B, S, N, H, D
+    p.B, p.S, p.N, p.H, p.D = B, S, N, H, _pad_head_dim(D)
     p.dtype = _DTYPES[Q.dtype]
     p.bias_dtype, p.mask_kind = _lib.EVO_NONE, _lib.EVO_MASK_NONE
     if pair_bias is not None:

@@ -536,6 +536,28 @@ def test_head_dim_128_on_the_matrix_core(E, case):
     assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_BWD) == b"mfma"
 
 
+@pytest.mark.parametrize("case", [(1, 3, 100, 2, 24, "bool", "q", "reference"), (2, 2, 256, 2, 48, "add", "q", "ds4sci"),
+                                  (1, 4, 130, 3, 96, "soft", torch.float32, "reference"), (1, 2, 64, 2, 4, None, None, "reference")],
+                         ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_head_dims_between_the_built_ones_are_padded(E, case):
+    """A head dim the library is not built for runs at the next one that it is, on zero columns, with
+    the caller's softmax scale; outputs and gradients come back in the caller's shape."""
+    B, S, N, H, D, mask, bias_dt, layout = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, torch.bfloat16, std=0.8)
+    ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, layout=layout, compute_dtype=torch.float32)
+    fmask = m is not None and m.dtype != torch.bool
+    got = run_hip(E, Q, K, V, m, bias, dO, layout=layout, mask_grad=fmask)
+    for n in ("O", "dQ", "dK", "dV"):
+        assert got[n].shape == Q.shape and got[n].is_contiguous()
+    assert_close(got, ref, BF16_TOL, ["O", "dQ", "dK", "dV", "dBias"] + (["dMask"] if fmask else []), what=str(case),
+                 ulp_names=("dQ", "dK", "dV", "dBias", "dMask"))
+    # the registered operators take the same route
+    dev = "cuda"
+    o, lse, _ = torch.ops.evoattn.fwd(Q.to(dev), K.to(dev), V.to(dev), None if m is None else m.to(dev),
+                                      None if bias is None else bias.to(dev), layout == "ds4sci")
+    assert torch.equal(o, got["O"]) and lse.shape == (B, H, S, N)
+
+
 def test_generic_fallbacks(E):
     """A 2-byte-aligned storage offset is served by the plain kernels."""
     Q, K, V, m, bias, dO = make_case(1, 2, 48, 2, 32, "add", "q", torch.bfloat16)

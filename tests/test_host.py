@@ -117,3 +117,12 @@ def test_registered_operators_schema_and_shape_only_implementations():
     x = torch.zeros(1, 2, 8, 2, 8)
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.evoattn.fwd(x, x, x, None, None, False)
+
+
+def test_head_dim_padding_rule():
+    assert [E._pad_head_dim(d) for d in (1, 8, 9, 16, 24, 32, 48, 64, 96, 128)] == [8, 8, 16, 16, 32, 32, 64, 64, 128, 128]
+    with pytest.raises(ValueError):
+        E._pad_head_dim(129)
+    x = torch.ones(2, 3, 24)
+    y = E._padded(x, 32)
+    assert y.shape == (2, 3, 32) and float(y[..., 24:].abs().sum()) == 0.0 and E._padded(x, 24) is x
