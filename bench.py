@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--preheat-seconds", type=float, default=1.0,
                     help="untimed steps before the warm-up steps until this much wall time has passed: the chip "
                          "takes some tenths of a second of load to reach its steady clocks, and a handful of "
-                         "400-microsecond warm-up steps ends before that (measured: 8 % slower steps)")
+                         "400-microsecond warm-up steps ends before that (measured: 8 %% slower steps)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bias", action="store_true",
                     help="the same shape without the pair bias (and so without dBias): the no-bias forms of the "
