@@ -158,6 +158,12 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
     _check_qkv(Q, K, V)
     lib = _lib.load()
     B, S, N, H, D = Q.shape
+    if Q.numel() == 0:          # no problem or no residue: nothing to launch (eager returns an empty tensor too)
+        mask_meta = (_lib.EVO_MASK_NONE, (0, 0), None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
+        bias_meta = (_lib.EVO_NONE, (0, 0, 0), None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+        return (Q.contiguous(), K.contiguous(), V.contiguous(), res_mask, pair_bias, torch.empty_like(Q.contiguous()),
+                torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32), _alloc_bytes(0, Q.device),
+                mask_meta, bias_meta)
     Dp = _pad_head_dim(D)
     Qc, Kc, Vc = Q.contiguous(), K.contiguous(), V.contiguous()
     Qp, Kp, Vp = _padded(Qc, Dp), _padded(Kc, Dp), _padded(Vc, Dp)
@@ -201,6 +207,13 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
     B, S, N, H, D = Q.shape
     mask_kind, mstr, mask_orig = mask_meta
     bias_dt, bstr, bias_orig = bias_meta
+    if Q.numel() == 0:          # empty problem: empty gradients, zeros for the bias and a floating mask
+        dmask = dbias = None
+        if need_dbias and bias is not None:
+            dbias = torch.zeros(bias_orig[0], device=Q.device, dtype=bias_orig[1])
+        if need_dmask and mask is not None and mask.is_floating_point():
+            dmask = torch.zeros(mask_orig[0], device=Q.device, dtype=mask_orig[1])
+        return torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V), dmask, dbias
     dO = dO.contiguous()                                        # the reference asserts this, :747
     if dO.dtype != Q.dtype:
         dO = dO.to(Q.dtype)

@@ -558,6 +558,25 @@ def test_head_dims_between_the_built_ones_are_padded(E, case):
     assert torch.equal(o, got["O"]) and lse.shape == (B, H, S, N)
 
 
+@pytest.mark.parametrize("shape", [(1, 0, 64, 2, 32), (2, 3, 0, 2, 16), (0, 2, 8, 1, 8)], ids=lambda s: "x".join(map(str, s)))
+def test_empty_inputs(E, shape):
+    """No S row, no residue or no batch entry: empty output and gradients (as the eager formula
+    gives), zeros for the bias gradient, nothing launched."""
+    B, S, N, H, D = shape
+    dev = "cuda"
+    q, k, v = (torch.zeros(shape, dtype=torch.bfloat16, device=dev, requires_grad=True) for _ in range(3))
+    m = torch.ones((B, S, 1, 1, N), dtype=torch.bool, device=dev)
+    b = torch.randn((B, 1, H, N, N), dtype=torch.bfloat16, device=dev, requires_grad=True)
+    o = E.EvoformerAttention.apply(q, k, v, m, b)
+    assert o.shape == q.shape and o.dtype == q.dtype
+    o.backward(torch.zeros_like(o))
+    torch.cuda.synchronize()
+    assert q.grad.shape == q.shape and k.grad.shape == q.shape and v.grad.shape == q.shape
+    assert b.grad.shape == b.shape and float(b.grad.float().abs().sum()) == 0.0
+    ref = eager.attention(q.detach().cpu(), k.detach().cpu(), v.detach().cpu(), m.cpu(), b.detach().cpu())
+    assert ref.shape == o.shape
+
+
 def test_generic_fallbacks(E):
     """A 2-byte-aligned storage offset is served by the plain kernels."""
     Q, K, V, m, bias, dO = make_case(1, 2, 48, 2, 32, "add", "q", torch.bfloat16)
