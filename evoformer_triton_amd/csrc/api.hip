@@ -40,6 +40,7 @@ static int check_common(const EvoAttnParams *p) {
 
 // The matrix-core kernels read rows with 16-byte loads and keep one 32-wide key tile per
 // 16 accumulator registers in the dBias kernel (at most 16 tiles per wave, 4 waves).
+static bool long_rows_bwd_ok(const EvoAttnParams &p);
 static bool mfma_ok(const EvoAttnParams &p, int pass) {
     if (p.flags & EVO_FLAG_FORCE_GENERIC) return false;
     if (p.dtype != EVO_BF16 && p.dtype != EVO_F16) return false;
@@ -47,7 +48,7 @@ static bool mfma_ok(const EvoAttnParams &p, int pass) {
     if (p.stride_b % 8 || p.stride_h % 8 || p.stride_s % 8 || p.stride_n % 8) return false;
     if (!aligned(p.q, 16) || !aligned(p.k, 16) || !aligned(p.v, 16) || !aligned(p.o, 16)) return false;
     if (pass == EVO_PASS_BWD) {
-        if (p.N > 2048) return false;
+        if (p.N > 2048 && !long_rows_bwd_ok(p)) return false;
         if (!aligned(p.dout, 16) || !aligned(p.dq, 16) || !aligned(p.dk, 16) || !aligned(p.dv, 16)) return false;
     }
     return true;
@@ -67,6 +68,9 @@ static int bias_vec_ok(const EvoAttnParams &p) {
 // keeps the tiles, for comparison.
 static bool bias_direct(const EvoAttnParams &p) {
     if (!p.bias || p.S > 4 || (p.flags & 0x800) || p.N % 4) return false;
+    // beyond 2048 keys a dBias summed over several S rows needs the kernel that reads prepared tiles
+    // (decided without looking at dbias: the forward, which prepares, has none)
+    if (p.N > 2048 && p.S > 1) return false;
     if (p.bias_dtype != EVO_F32 && p.bias_dtype != p.dtype) return false;
     if ((int64_t)p.N * p.bias_stride_row >= ((int64_t)1 << 31)) return false;   // 32-bit offsets inside one (b, h) matrix
     return bias_vec_ok(p) != 0;
@@ -104,7 +108,7 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     // prefetch (head dim 64 beyond 128 keys) or measured slower
     // fewest S rows: the second kernel's start-up has to pay (N = 768, D = 32: ahead from 8 rows on;
     // N = 512: 72 against 66 us at 32 rows)
-    const int min_s = p.D == 32 && p.N > 512 ? 8 : 64;
+    const int min_s = p.N > 2048 ? 2 : p.D == 32 && p.N > 512 ? 8 : 64;   // (beyond 2048 keys the one kernel has no form at all)
     const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
     if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
@@ -114,6 +118,11 @@ static bool dq_split_ok(const EvoAttnParams &p) {
 static bool dq_wide_ok(const EvoAttnParams &p) {
     return dq_wide_grid_ok(p) && (!p.dbias || p.S == 1 || dq_split_ok(p));
 }
+// Rows of more than 2048 keys: the dQ kernels that keep the dBias sums of a wave's key tiles in
+// registers have no form that long (16 tiles per wave would be the whole register file).  The
+// backward still runs on the matrix core where dQ comes from the kernel without those sums:
+// no dBias asked for, S = 1, or the dBias kernel of its own (bias in the dtype of q).
+static bool long_rows_bwd_ok(const EvoAttnParams &p) { return dq_wide_ok(p); }
 static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && p.S == 1 && dq_wide_ok(p); }
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and

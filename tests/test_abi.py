@@ -124,6 +124,12 @@ def test_path_selection(lib):
     p = good(N=4096)
     assert lib.evoattn_path(ctypes.byref(p), 0) == b"mfma"
     assert lib.evoattn_path(ctypes.byref(p), 1) == b"generic"            # dBias tiles exceed the register file
+    p.bias_dtype = p.dbias_dtype = _lib.EVO_BF16                           # ... unless a kernel of its own sums dBias
+    assert lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
+    assert lib.evoattn_kernels(ctypes.byref(p), 1) == b"mfma_dq_wide+mfma_dbias,mfma_dkdv"
+    p = good(N=4096)
+    p.dbias = None
+    assert lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
 
 
 def test_error_strings(lib):

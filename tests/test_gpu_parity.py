@@ -577,6 +577,49 @@ def test_empty_inputs(E, shape):
     assert ref.shape == o.shape
 
 
+LONG_ROWS = [  # B, S, N, H, D, mask, bias dtype, dBias asked for, backward on the matrix core
+    (1, 2, 2304, 1, 32, "bool", "q", True, True),              # dQ without the sums + the dBias kernel of its own
+    (1, 1, 2304, 2, 64, "add", "q", True, True),               # S = 1: dBias written by the dQ kernel
+    (1, 2, 2560, 1, 16, "bool", None, False, True),            # no bias
+    (1, 3, 2304, 1, 32, "soft", torch.float32, False, True),   # bias as a constant
+    (1, 2, 2304, 1, 32, "bool", torch.float32, True, False),   # fp32 bias with a gradient: the plain kernels
+]
+
+
+@pytest.mark.parametrize("case", LONG_ROWS, ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
+def test_rows_beyond_2048_keys(E, case):
+    """The backward of rows longer than 2048 keys runs on the matrix core wherever dQ can come from the
+    kernel that keeps no dBias sums (`evoattn_path` through the C ABI says which), and meets the bound."""
+    from evoformer_triton_amd import _lib
+    B, S, N, H, D, mask, bias_dt, bias_grad, on_mfma = case
+    Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, torch.bfloat16, seed=91, std=0.7)
+    dev = "cuda"
+    on = lambda t: None if t is None else t.to(dev)
+    ref = eager.attention_fwd_bwd(on(Q), on(K), on(V), on(m), on(bias), on(dO), compute_dtype=torch.float32, s_chunk=1)
+    q, k, v = (t.to(dev).requires_grad_() for t in (Q, K, V))
+    b = on(bias)
+    if b is not None and bias_grad:
+        b.requires_grad_()
+    o = E.EvoformerAttention.apply(q, k, v, on(m), b)
+    o.backward(on(dO))
+    torch.cuda.synchronize()
+    got = {"O": o.detach(), "dQ": q.grad, "dK": k.grad, "dV": v.grad}
+    names = ["O", "dQ", "dK", "dV"]
+    if b is not None and bias_grad:
+        got["dBias"] = b.grad
+        names.append("dBias")
+    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+    lib = _lib.load()
+    mm, mk, mstr = E._prep_mask(on(m), B, S, N, q.device)
+    bb, bdt, bstr = E._prep_bias(b, B, H, N, q.dtype, q.device)
+    p = E._params(q.detach(), k.detach(), v.detach(), mm, mk, mstr, bb, bdt, bstr, torch.empty_like(q),
+                  torch.empty((B, H, S, N), device=dev), "reference")
+    p.dout, p.dq, p.dk, p.dv = (ctypes.c_void_p(t.data_ptr()) for t in (q.grad, q.grad, k.grad, v.grad))
+    if b is not None and bias_grad:
+        p.dbias, p.dbias_dtype = ctypes.c_void_p(b.grad.data_ptr()), E._DTYPES[b.dtype]
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_BWD) == (b"mfma" if on_mfma else b"generic")
+
+
 def test_generic_fallbacks(E):
     """A 2-byte-aligned storage offset is served by the plain kernels."""
     Q, K, V, m, bias, dO = make_case(1, 2, 48, 2, 32, "add", "q", torch.bfloat16)
