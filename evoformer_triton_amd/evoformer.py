@@ -187,8 +187,8 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
 def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
     if torch.compiler.is_compiling():
         # under torch.compile the device work is the registered operator (opaque to the tracer)
-        O, lse, prep = torch.ops.evoattn.fwd(Q, K, V, res_mask, pair_bias, layout == "ds4sci")
-        ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep)
+        O, lse, prep, seen = torch.ops.evoattn.fwd(Q, K, V, res_mask, pair_bias, layout == "ds4sci")
+        ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep, seen)
         ctx.layout, ctx.through_ops = layout, True
         return O
     Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta = _fwd_impl(Q, K, V, res_mask, pair_bias, layout)
@@ -263,8 +263,8 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
 
 def _backward(ctx, dO, need_dmask, need_dbias):
     if ctx.through_ops:
-        Q, K, V, res_mask, pair_bias, O, lse, prep = ctx.saved_tensors
-        dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep,
+        Q, K, V, res_mask, pair_bias, O, lse, prep, seen = ctx.saved_tensors
+        dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, seen,
                                                          ctx.layout == "ds4sci", bool(need_dbias), bool(need_dmask))
         want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
         return dQ, dK, dV, (dmask if want_dmask else None), (dbias if need_dbias and pair_bias is not None else None)
@@ -279,11 +279,19 @@ def _backward(ctx, dO, need_dmask, need_dbias):
 
 @torch.library.custom_op("evoattn::fwd", mutates_args=(), device_types="cuda")
 def _op_fwd(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
-            pair_bias: Optional[torch.Tensor], per_head: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(O, LSE [B,H,S,N] fp32, prep bytes): the forward of EvoformerAttention (per_head False:
-    the reference's flat-reshape heads) or of DS4Sci_EvoformerAttention (per_head True)."""
+            pair_bias: Optional[torch.Tensor], per_head: bool
+            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(O, LSE [B,H,S,N] fp32, prep bytes, seen): the forward of EvoformerAttention (per_head
+    False: the reference's flat-reshape heads) or of DS4Sci_EvoformerAttention (per_head True).
+    `seen` (two int64 on the CPU) holds the addresses of the mask and the bias the kernels read:
+    the backward reuses the prepared bytes only if it is handed the same memory."""
     out = _fwd_impl(Q, K, V, res_mask, pair_bias, "ds4sci" if per_head else "reference", prep_upper=True)
-    return out[5], out[6], out[7]
+    return out[5], out[6], out[7], _seen(out[3], out[4])
+
+
+def _seen(mask, bias):
+    return torch.tensor([0 if mask is None else mask.data_ptr(), 0 if bias is None else bias.data_ptr()],
+                        dtype=torch.int64)
 
 
 @_op_fwd.register_fake
@@ -304,13 +312,13 @@ def _(Q, K, V, res_mask, pair_bias, per_head):
         p.mask_kind = _lib.EVO_MASK_BOOL if not res_mask.is_floating_point() else _MASK_KINDS.get(res_mask.dtype, _lib.EVO_MASK_F32)
     nbytes = max(int(lib.evoattn_prep_bytes(ctypes.byref(p))), 256)
     return (Q.new_empty(Q.shape), Q.new_empty((B, H, S, N), dtype=torch.float32),
-            Q.new_empty((nbytes,), dtype=torch.uint8))
+            Q.new_empty((nbytes,), dtype=torch.uint8), torch.empty((2,), dtype=torch.int64, device="cpu"))
 
 
 @torch.library.custom_op("evoattn::bwd", mutates_args=(), device_types="cuda")
 def _op_bwd(dO: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
             pair_bias: Optional[torch.Tensor], O: torch.Tensor, lse: torch.Tensor, prep: torch.Tensor,
-            per_head: bool, need_dbias: bool, need_dmask: bool
+            seen: torch.Tensor, per_head: bool, need_dbias: bool, need_dmask: bool
             ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dQ, dK, dV, dMask, dBias) from the forward's inputs and outputs; a gradient that was not
     asked for (or has no tensor to belong to) comes back as an empty tensor."""
@@ -320,8 +328,9 @@ def _op_bwd(dO: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
     bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
     mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
-    # the prepared tiles are the forward's only if the kernels read the very same tensors
-    same = mask is res_mask and bias is pair_bias
+    # the prepared bytes are the forward's only if the kernels read the very same memory (a traced
+    # graph may hand the backward a recomputed copy, whose alignment decides the layout anew)
+    same = bool(torch.equal(seen.cpu(), _seen(mask, bias)))
     dQ, dK, dV, dmask, dbias = _bwd_impl(dO, Qc, Kc, Vc, mask, bias, O.contiguous(), lse, prep,
                                          "ds4sci" if per_head else "reference", mask_meta, bias_meta,
                                          need_dmask, need_dbias, prep_valid=same)
@@ -330,7 +339,7 @@ def _op_bwd(dO: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
 
 
 @_op_bwd.register_fake
-def _(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, per_head, need_dbias, need_dmask):
+def _(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, seen, per_head, need_dbias, need_dmask):
     want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
     want_dbias = need_dbias and pair_bias is not None
     return (Q.new_empty(Q.shape), Q.new_empty(Q.shape), Q.new_empty(Q.shape),
@@ -340,16 +349,16 @@ def _(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, per_head, need_dbias, need
 
 def _op_setup_context(ctx, inputs, output):
     Q, K, V, res_mask, pair_bias, per_head = inputs
-    O, lse, prep = output
-    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep)
+    O, lse, prep, seen = output
+    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, O, lse, prep, seen)
     ctx.per_head = per_head
 
 
-def _op_backward(ctx, dO, dlse, dprep):
-    Q, K, V, res_mask, pair_bias, O, lse, prep = ctx.saved_tensors
+def _op_backward(ctx, dO, dlse, dprep, dseen):
+    Q, K, V, res_mask, pair_bias, O, lse, prep, seen = ctx.saved_tensors
     need_dmask = bool(ctx.needs_input_grad[3] and res_mask is not None and res_mask.is_floating_point())
     need_dbias = bool(ctx.needs_input_grad[4] and pair_bias is not None)
-    dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep,
+    dQ, dK, dV, dmask, dbias = torch.ops.evoattn.bwd(dO, Q, K, V, res_mask, pair_bias, O, lse, prep, seen,
                                                      ctx.per_head, need_dbias, need_dmask)
     return dQ, dK, dV, (dmask if need_dmask else None), (dbias if need_dbias else None), None
 

@@ -553,7 +553,7 @@ def test_head_dims_between_the_built_ones_are_padded(E, case):
                  ulp_names=("dQ", "dK", "dV", "dBias", "dMask"))
     # the registered operators take the same route
     dev = "cuda"
-    o, lse, _ = torch.ops.evoattn.fwd(Q.to(dev), K.to(dev), V.to(dev), None if m is None else m.to(dev),
+    o, lse, _, _ = torch.ops.evoattn.fwd(Q.to(dev), K.to(dev), V.to(dev), None if m is None else m.to(dev),
                                       None if bias is None else bias.to(dev), layout == "ds4sci")
     assert torch.equal(o, got["O"]) and lse.shape == (B, H, S, N)
 
@@ -765,7 +765,7 @@ def test_registered_operators_match_the_function(E, case):
     mm = None if m is None else m.to(dev)
     if fmask:
         mm.requires_grad_()
-    o, lse, _ = torch.ops.evoattn.fwd(q, k, v, mm, b, per_head)
+    o, lse, _, _ = torch.ops.evoattn.fwd(q, k, v, mm, b, per_head)
     o.backward(dO.to(dev))
     torch.cuda.synchronize()
     assert lse.shape == (B, H, S, N) and lse.dtype == torch.float32
@@ -777,6 +777,26 @@ def test_registered_operators_match_the_function(E, case):
         assert torch.equal(mm.grad, plain["dMask"])
 
 
+def test_backward_operator_handed_a_copy_of_the_bias_prepares_again(E):
+    """A traced graph may recompute a cheap producer of the bias in the backward: the backward operator then
+    sees other memory (here at another alignment, which changes the layout of the prepared bytes for few S rows)
+    and must not trust what the forward prepared."""
+    Q, K, V, m, bias, dO = make_case(2, 2, 100, 2, 32, "bool", "q", torch.bfloat16)
+    plain = run_hip(E, Q, K, V, m, bias, dO)
+    dev = "cuda"
+    q, k, v, mm, b, g = (t.to(dev) for t in (Q, K, V, m, bias, dO))
+    o, lse, prep, seen = torch.ops.evoattn.fwd(q, k, v, mm, b, False)
+    buf = torch.empty(b.numel() + 1, dtype=b.dtype, device=dev)
+    buf[1:] = b.reshape(-1)
+    b2 = buf[1:].view(b.shape)                       # same values, 2-byte aligned
+    assert b2.data_ptr() % 16 != 0
+    dq, dk, dv, _, db = torch.ops.evoattn.bwd(g, q, k, v, mm, b2, o, lse, prep, seen, False, True, False)
+    torch.cuda.synchronize()
+    assert torch.equal(o, plain["O"])
+    for a, w in ((dq, "dQ"), (dk, "dK"), (dv, "dV"), (db, "dBias")):
+        assert max_err(a, plain[w]) <= 1e-6 + 2.0 ** -7 * plain[w].float().abs().max().item(), w
+
+
 def test_registered_operators_pass_opcheck(E):
     """Schema, shape-only implementation and autograd registration, as torch.library checks them."""
     Q, K, V, m, bias, dO = make_case(1, 3, 64, 2, 32, "bool", "q", torch.bfloat16)
@@ -786,9 +806,9 @@ def test_registered_operators_pass_opcheck(E):
     tests = ("test_schema", "test_faketensor", "test_autograd_registration")
     torch.library.opcheck(torch.ops.evoattn.fwd, (q, k, v, m.to(dev), b, False), test_utils=tests)
     with torch.no_grad():
-        o, lse, prep = torch.ops.evoattn.fwd(q, k, v, m.to(dev), b, False)
+        o, lse, prep, seen = torch.ops.evoattn.fwd(q, k, v, m.to(dev), b, False)
     torch.library.opcheck(torch.ops.evoattn.bwd, (dO.to(dev), q.detach(), k.detach(), v.detach(), m.to(dev), b.detach(),
-                                                  o, lse, prep, False, True, False), test_utils=tests[:2])
+                                                  o, lse, prep, seen, False, True, False), test_utils=tests[:2])
 
 
 @pytest.mark.parametrize("case", [(1, 6, 256, 2, 32, "add", "q"), (2, 3, 100, 2, 16, "bool", torch.float32)],

@@ -98,21 +98,22 @@ def test_registered_operators_schema_and_shape_only_implementations():
     from torch._subclasses.fake_tensor import FakeTensorMode
     assert str(torch.ops.evoattn.fwd.default._schema) == (
         "evoattn::fwd(Tensor Q, Tensor K, Tensor V, Tensor? res_mask, Tensor? pair_bias, bool per_head)"
-        " -> (Tensor, Tensor, Tensor)")
+        " -> (Tensor, Tensor, Tensor, Tensor)")
     assert "bool need_dbias, bool need_dmask" in str(torch.ops.evoattn.bwd.default._schema)
     B, S, N, H, D = 2, 3, 100, 4, 16
     with FakeTensorMode():
         q = torch.empty(B, S, N, H, D, device="cuda", dtype=torch.bfloat16)
         m = torch.empty(1, S, 1, 1, N, device="cuda", dtype=torch.float16)
         b = torch.empty(1, 1, H, N, N, device="cuda", dtype=torch.float32)
-        o, lse, prep = torch.ops.evoattn.fwd(q, q, q, m, b, False)
+        o, lse, prep, seen = torch.ops.evoattn.fwd(q, q, q, m, b, False)
+        assert seen.device.type == "cpu" and seen.dtype == torch.int64 and seen.shape == (2,)
         assert o.shape == q.shape and o.dtype == q.dtype and o.is_contiguous()
         assert lse.shape == (B, H, S, N) and lse.dtype == torch.float32
         assert prep.dtype == torch.uint8 and prep.numel() >= 256
-        dq, dk, dv, dm, db = torch.ops.evoattn.bwd(o, q, q, q, m, b, o, lse, prep, False, True, True)
+        dq, dk, dv, dm, db = torch.ops.evoattn.bwd(o, q, q, q, m, b, o, lse, prep, seen, False, True, True)
         assert dq.shape == dk.shape == dv.shape == q.shape
         assert dm.shape == m.shape and dm.dtype == m.dtype and db.shape == b.shape and db.dtype == b.dtype
-        dq, dk, dv, dm, db = torch.ops.evoattn.bwd(o, q, q, q, None, b, o, lse, prep, True, False, True)
+        dq, dk, dv, dm, db = torch.ops.evoattn.bwd(o, q, q, q, None, b, o, lse, prep, seen, True, False, True)
         assert dm.numel() == 0 and db.numel() == 0
     x = torch.zeros(1, 2, 8, 2, 8)
     with pytest.raises((NotImplementedError, RuntimeError)):
