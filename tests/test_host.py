@@ -82,7 +82,9 @@ def test_argument_errors_and_no_cpu_fallback():
 
 def test_drop_in_module_name():
     import evoformer
+    import unmasked_evoformer
     assert evoformer.EvoformerAttention is E.EvoformerAttention
+    assert unmasked_evoformer.EvoformerAttention is E.EvoformerAttention
 
 
 def test_missing_library_fails_loudly(tmp_path):
