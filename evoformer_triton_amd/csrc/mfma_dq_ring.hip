@@ -101,6 +101,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar, so that what depends on it branches
+    __builtin_assume(wave >= 0 && wave < 8);                     // (512 threads: lets piece numbers be bounded at compile time)
     const int li = lane & 31, g = lane >> 5;
     const int qi = wave / KQ, kq = wave % KQ;
     const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
