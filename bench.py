@@ -46,7 +46,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", default="C2", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--config", default="C2", choices=["C1", "C2", "C3", "C4", "C5"],
+                    help="C2 is the headline workload; C1 is the small fp32 case (the all-fp32 check mode of the library "
+                         "beside the same eager formula on the host CPU), C3-C5 the other benchmark configurations")
     ap.add_argument("--preheat-seconds", type=float, default=1.0,
                     help="untimed steps before the warm-up steps until this much wall time has passed: the chip "
                          "takes some tenths of a second of load to reach its steady clocks, and a handful of "
@@ -161,7 +163,7 @@ def cpu_baseline(cfg, shape, budget_s=15.0, with_bias=True):
     from oracle import eager
     B, S, N, H, D = shape
     threads = torch.get_num_threads()
-    s_sample = S if cfg in ("C2", "C3") else max(1, S // 8)   # whole workload where it takes well under a second
+    s_sample = S if cfg in ("C1", "C2", "C3") else max(1, S // 8)   # whole workload where it takes well under a second
     x = eager.make_inputs(cfg, shape=(B, s_sample, N, H, D))
 
     def once():
@@ -176,7 +178,7 @@ def cpu_baseline(cfg, shape, budget_s=15.0, with_bias=True):
     flops = eager.flops_fwd_bwd(B, s_sample, N, H, D)[2]
     return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"{s_sample} of {S} S-rows of {cfg} ({s_sample / S:.4f} of the workload), eager fp32 oracle "
-                      f"chunked 8 rows at a time, 1 warm-up + median of {reps} runs, {t:.3f} s per run"}
+                      f"chunked 8 rows at a time, 1 warm-up + median of {reps} runs, {t * 1e3:.2f} ms per run"}
 
 
 def main():
@@ -288,7 +290,8 @@ def main():
     achieved = phases[dom][1] / t_phase[dom] / 1e12
     p.flags = 0
     k_fwd = lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_FWD).decode()
-    k_dq, k_dkdv = lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().split(",")
+    k_bwd = lib.evoattn_kernels(ctypes.byref(p), _lib.EVO_PASS_BWD).decode().split(",")
+    k_dq, k_dkdv = (k_bwd[0] + " (dQ)", k_bwd[0] + " (dK/dV)") if len(k_bwd) == 1 else k_bwd
     kernel_names = {"fwd": "prep_kernel+" + k_fwd, "bwd_dq": k_dq, "bwd_dkdv": k_dkdv}
     if args.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
@@ -317,11 +320,11 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": {torch.bfloat16: "bf16", torch.float16: "fp16", torch.float32: "f32"}[qc.dtype],
         "data": "synthetic",
         "config": {"workload": f"{args.config}: Evoformer attention fwd+bwd through EvoformerAttention.apply + autograd, "
-                               f"Q,K,V [B={B},S={S},N={N},H={H},D={D}] bf16, additive row mask [{B},{S},1,1,{N}], "
-                               + ("no pair bias" if bias is None else f"pair bias [{B},1,{H},{N},{N}] bf16") + ", seeded N(0,1) inputs",
+                               f"Q,K,V [B={B},S={S},N={N},H={H},D={D}] {str(qc.dtype)[6:]}, additive row mask [{B},{S},1,1,{N}], "
+                               + ("no pair bias" if bias is None else f"pair bias [{B},1,{H},{N},{N}] {str(bias.dtype)[6:]}") + ", seeded N(0,1) inputs",
                    "flops_per_step": f_full, "algorithmic_hbm_bytes_per_step": io_bytes},
         "pct_mfma_peak": 100.0 * f_full / dt / 1e12 / MFMA_PEAK_TFLOPS,
         "pct_hbm_peak": 100.0 * io_bytes / dt / 1e9 / HBM_PEAK_GBS,
