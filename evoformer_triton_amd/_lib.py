@@ -19,6 +19,10 @@ EVO_FLAG_PREP_VALID = 2
 EVO_FLAG_ONLY_DQ = 4
 EVO_FLAG_ONLY_DKDV = 8
 EVO_FLAG_PER_PROBLEM = 16
+EVO_FLAG_DEBUG_NO_KV_RING = 0x200
+EVO_FLAG_DEBUG_BIAS_TILES = 0x800
+EVO_FLAG_DEBUG_NO_DQ_WIDE = 0x1000
+EVO_FLAG_DEBUG_NO_DQ_SPLIT = 0x2000
 EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 

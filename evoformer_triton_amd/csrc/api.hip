@@ -1,6 +1,8 @@
 // C ABI of the library: parameter validation, workspace layout and kernel dispatch.
 // Everything in this file runs on the host; nothing here needs a GPU except the two
 // enqueue entry points.
+#include <atomic>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -20,6 +22,7 @@ static int check_common(const EvoAttnParams *p) {
     if ((p->mask_kind == EVO_MASK_NONE) != (p->mask == nullptr)) return EVO_EINVAL;
     if (!p->q || !p->k || !p->v || !p->o || !p->lse) return EVO_EINVAL;
     if (!(p->scale == p->scale) || p->scale <= 0.0f) return EVO_EINVAL;
+    if (p->flags & ~EVO_FLAG_ALL) return EVO_EINVAL;
     if (p->D != 8 && p->D != 16 && p->D != 32 && p->D != 64 && p->D != 128) return EVO_EUNSUPPORTED;
     if (p->stride_b < 0 || p->stride_h < 0 || p->stride_s < 0 || p->stride_n < p->D) return EVO_EINVAL;
     if (p->bias && (p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_row < p->N)) return EVO_EINVAL;
@@ -64,10 +67,9 @@ static int bias_vec_ok(const EvoAttnParams &p) {
 // per bias entry before any kernel has used one; each kernel then reads 4 bytes per entry and S
 // row.  With very few S rows per (batch, head) - the reference's own speed benchmark has one -
 // the one-workgroup-per-problem kernels read the caller's tensor instead, which needs rows that
-// allow 16-byte (fp32) or 8-byte loads.  Bit 0x800 of flags (not part of the public interface)
-// keeps the tiles, for comparison.
+// allow 16-byte (fp32) or 8-byte loads.  EVO_FLAG_DEBUG_BIAS_TILES keeps the tiles, for comparison.
 static bool bias_direct(const EvoAttnParams &p) {
-    if (!p.bias || p.S > 4 || (p.flags & 0x800) || p.N % 4) return false;
+    if (!p.bias || p.S > 4 || (p.flags & EVO_FLAG_DEBUG_BIAS_TILES) || p.N % 4) return false;
     // beyond 2048 keys a dBias summed over several S rows needs the kernel that reads prepared tiles
     // (decided without looking at dbias: the forward, which prepares, has none)
     if (p.N > 2048 && p.S > 1) return false;
@@ -87,10 +89,9 @@ static bool dq_ring_ok(const EvoAttnParams &p) {
 // S = 1 writes dBias as it goes (no partials, no reduction).  Its workgroups take 128 query
 // rows each and walk over the keys one tile after the other: with very few of them the
 // kernels that split a row's keys over the waves finish sooner (N = 300, 6 workgroups: 10.4 us
-// against 8.2 us).  Bit 0x1000 of flags (not part of the public interface) selects the other
-// kernels, for comparison.
+// against 8.2 us).  EVO_FLAG_DEBUG_NO_DQ_WIDE selects the other kernels, for comparison.
 static bool dq_wide_grid_ok(const EvoAttnParams &p) {
-    return !(p.flags & (EVO_FLAG_PER_PROBLEM | 0x1000)) && (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
+    return !(p.flags & (EVO_FLAG_PER_PROBLEM | EVO_FLAG_DEBUG_NO_DQ_WIDE)) && (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
 }
 
 // Rows of more than 384 keys with a dBias to sum (up to there the dQ kernel that keeps the sums
@@ -102,7 +103,7 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 // 1.56 ms; N = 384: 211 against 204 us, and with few S rows the second kernel's start-up shows;
 // head dims 8 and 16, whose one-kernel form reaches to N = 512: 569 against 367 us and 696
 // against 661 us there, 0.65 against 1.38 ms and 740 against 793 us at N = 768).
-// Bit 0x2000 of flags (not part of the public interface) selects the one kernel, for comparison.
+// EVO_FLAG_DEBUG_NO_DQ_SPLIT selects the one kernel, for comparison.
 static bool dq_split_ok(const EvoAttnParams &p) {
     // shortest rows that go this way: where the kernel that keeps the sums has no form with
     // prefetch (head dim 64 beyond 128 keys) or measured slower
@@ -111,7 +112,7 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     const int min_s = p.N > 2048 ? 2 : p.D == 32 && p.N > 512 ? 8 : 64;   // (beyond 2048 keys the one kernel has no form at all)
     const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
     if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
-    if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & 0x2000) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
+    if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }
 
@@ -308,10 +309,10 @@ static bool fwd_ring_ok(const EvoAttnParams &p) {
 }
 
 // The dK/dV kernel that walks over a chunk of S rows keeps 16-bit bias columns resident: it
-// takes a bias in the dtype of q (or none) and rows whose length is a multiple of 8.  Bit
-// 0x200 of flags (not part of the public interface) selects the other kernel, for comparison.
+// takes a bias in the dtype of q (or none) and rows whose length is a multiple of 8.  
+// EVO_FLAG_DEBUG_NO_KV_RING selects the other kernel, for comparison.
 static bool kv_ring_ok(const EvoAttnParams &p) {
-    if ((p.flags & (EVO_FLAG_PER_PROBLEM | 0x200)) || p.N <= 128 || p.N > mfma_kvr_max_n(p.D) || p.N % 8) return false;
+    if ((p.flags & (EVO_FLAG_PER_PROBLEM | EVO_FLAG_DEBUG_NO_KV_RING)) || p.N <= 128 || p.N > mfma_kvr_max_n(p.D) || p.N % 8) return false;
     if (!aligned(p.lse, 16) || bias_direct(p)) return false;   // LSE rows are read four values at a time
     return !p.bias || p.bias_dtype == p.dtype;
 }
@@ -338,19 +339,24 @@ const char *evoattn_kernels(const EvoAttnParams *p, int pass) {
     return dq_ring_ok(*p) ? "mfma_dq_ring,mfma_dkdv" : "mfma_dq,mfma_dkdv";
 }
 
+// the forward's launches for a checked parameter block whose `prep` is in place
+static int fwd_launches(const EvoAttnParams &p, hipStream_t st) {
+    Extra e{};
+    e.vec_ok = bias_vec_ok(p);
+    fill_prep(p, e);
+    EVO_SET_TRACE(e);
+    if (const int rc = launch_prep(p, e, st)) return rc;
+    if (fwd_ring_ok(p)) return launch_mfma_fwdr(p, e, st);
+    return launch_mfma_fwd(p, e, st);
+}
+
 int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     int rc = evoattn_check(p, EVO_PASS_FWD);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)hip_stream;
     if (!mfma_ok(*p, EVO_PASS_FWD)) return launch_generic_fwd(*p, st);
     if ((rc = check_prep(*p))) return rc;
-    Extra e{};
-    e.vec_ok = bias_vec_ok(*p);
-    fill_prep(*p, e);
-    EVO_SET_TRACE(e);
-    if ((rc = launch_prep(*p, e, st))) return rc;
-    if (fwd_ring_ok(*p)) return launch_mfma_fwdr(*p, e, st);
-    return launch_mfma_fwd(*p, e, st);
+    return fwd_launches(*p, st);
 }
 
 int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {

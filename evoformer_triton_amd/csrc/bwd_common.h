@@ -1,6 +1,8 @@
 // Pieces shared by the backward matrix-core kernels of one head dim.
 #pragma once
 
+#include <atomic>
+
 #include "common.h"
 
 namespace evo {
@@ -51,25 +53,25 @@ __device__ __forceinline__ uint2 ones3() {
 
 // Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
 // copy of the kernel) and reports that device's CU count.  `done` is the caller's per-kernel
-// state, one slot per device ordinal.
+// state, one slot per device ordinal.  Host threads may make a kernel's first call on a device
+// at the same time: the slot is published with release / acquire ordering after the attribute
+// is set, and a thread that loses the race sets the same attribute to the same value again.
 constexpr int kMaxDevices = 64;
 struct PerDevice {
-    bool set[kMaxDevices];
-    int cus[kMaxDevices];
+    std::atomic<int> cus[kMaxDevices];   // 0: not set up yet on that device
 };
 static inline int ensure_dynamic_lds(const void *kern, int bytes, PerDevice &done, int *cus) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
     if (dev < 0 || dev >= kMaxDevices) return EVO_EUNSUPPORTED;
-    if (!done.set[dev]) {
-        int n = 0;
+    int n = done.cus[dev].load(std::memory_order_acquire);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
         const hipError_t err = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         if (err != hipSuccess) return EVO_EHIP - (int)err;
-        done.cus[dev] = n;
-        done.set[dev] = true;
+        done.cus[dev].store(n, std::memory_order_release);
     }
-    if (cus) *cus = done.cus[dev];
+    if (cus) *cus = n;
     return EVO_OK;
 }
 

@@ -26,7 +26,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 // A problem whose every key has a mask value below this is shifted by its largest mask
 // value so that the log-sum-exp keeps its mantissa.
-constexpr float kShiftThreshold = -1.0e5f;
+constexpr float kShiftThreshold = EVOATTN_SHIFT_THRESHOLD;
 // Most negative additive mask value the matrix-core kernels carry (in log2 units).
 constexpr float kMaskFloor = -1.0e30f;
 

@@ -22,10 +22,15 @@ __device__ __forceinline__ float row_shift(const EvoAttnParams &p, int b, int s)
     return shift_from_max(mx);
 }
 
+// A row whose every key is masked below the shift threshold (shift != 0) takes its scores from the
+// mask alone, as in the matrix-core kernels (prep.hip zeroes Q and the bias of such a row): the
+// two families may serve the forward and the backward of one call, and the backward's
+// exp(score - lse) is normalised only if both form the score the same way.  (Eager fp32
+// arithmetic does the same by rounding once the mask is large enough to swamp q.k + bias.)
 template <int BIASK, typename T>
 __device__ __forceinline__ float score(const EvoAttnParams &p, float qk, int64_t bias_off, float mk, float shift) {
-    float t = fmaf(qk, p.scale, load_bias1<BIASK, T>(p.bias, bias_off)) + mk;
-    return shift != 0.0f ? t - shift : t;
+    if (shift != 0.0f) return mk - shift;
+    return fmaf(qk, p.scale, load_bias1<BIASK, T>(p.bias, bias_off)) + mk;
 }
 
 template <typename T, int D, int BIASK>

@@ -18,10 +18,10 @@
 //
 // dBias is the sum of dS over S.  The reference adds every fp32 dS tile into global memory
 // with atomics (:458).  Here the dQ kernel owns a 32-query slab of one head for a whole
-// chunk of S rows and keeps the running sum of dS for that slab in matrix-core
-// accumulators (an identity-matrix MFMA adds the dS tile, rounded to fp16 for this purpose:
-// 11 significant bits per term, fp32 sum), writes one partial per chunk, and a second
-// kernel adds the partials in a fixed order: no floating-point atomics, bit-reproducible.
+// chunk of S rows and keeps the running sum of dS for that slab in registers (fp32
+// additions of the fp32 dS, as the reference adds fp32 dS at :456-459), writes one partial
+// per chunk, and a second kernel adds the partials in a fixed order: no floating-point
+// atomics, bit-reproducible.
 #include "bwd_common.h"
 #include "kernels.h"
 
@@ -36,7 +36,7 @@ namespace evo {
 // Workgroup = 4 waves = (b, h, chunk of S, 32 query rows).  The waves split the keys:
 // wave w takes 32-key tiles w, w+4, w+8, ...  Scores are computed transposed
 // (S^T = K Q^T, dP^T = V dO^T) so that a lane owns one query and 16 keys, which makes the
-// dS^T accumulator tile the B operand of both dQ^T += K^T dS^T and dBias^T += I dS^T.
+// dS^T accumulator tile the B operand of dQ^T += K^T dS^T and lines up with the dBias^T sums.
 // Each wave's partial dQ^T meets the others in LDS once per S row and is summed in wave
 // order.  Query slab and head are fixed for the whole S loop, so for N <= 512 the bias
 // tiles stay in registers across it.  delta = rowsum(dO * O) (evoformer.py:313-323) is
@@ -72,14 +72,6 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
     // rows d >= D of the transposed K tile are read by the MFMA but never written
     if (DP > D)
         for (int i = lane; i < (DP - D) * KTP; i += 64) Ktw[D * KTP + i] = (T)0.0f;
-
-    // identity slices in fp16: A[m][8g+i] = 1 where m is the key row that register 8ts+i of
-    // an accumulator tile holds for lane group g
-    f16x8 idf[2];
-#pragma unroll
-    for (int ts = 0; ts < 2; ++ts)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) idf[ts][i] = (f16_t)(li == crow(8 * ts + i, g) ? 1.0f : 0.0f);
 
     f32x16 dbacc[NTW];
 #pragma unroll
@@ -223,23 +215,23 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) ds[r] = 0.0f;
                 }
+                if (want_dbias) {
+                    // fp32 sums of the fp32 dS (compare chain: a static register index for a run-time tile number)
+#pragma unroll
+                    for (int jj = 0; jj < NTW; ++jj)
+                        if (jj == j) {
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) dbacc[jj][r] += ds[r];
+                        }
+                }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
                 for (int ts = 0; ts < 2; ++ts) {
                     v8 dsf;
-                    f16x8 dsh;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        dsf[i] = (T)ds[8 * ts + i];
-                        dsh[i] = (f16_t)ds[8 * ts + i];
-                    }
-                    if (want_dbias) {
-#pragma unroll
-                        for (int jj = 0; jj < NTW; ++jj)
-                            if (jj == j) dbacc[jj] = Mfma<f16_t>::mma(idf[ts], dsh, dbacc[jj]);
-                    }
+                    for (int i = 0; i < 8; ++i) dsf[i] = (T)ds[8 * ts + i];
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
                         v8 kta = *reinterpret_cast<const v8 *>(&Ktw[(dt * 32 + li) * KTP + ts * 16 + g * 8]);

@@ -62,8 +62,18 @@ enum {
     EVO_FLAG_ONLY_DKDV     = 8,
     /* Measurement aid: run the one-workgroup-per-(b,h,s) forms of the forward and dQ kernels
      * also where the forms that walk over a chunk of S rows apply (same results). */
-    EVO_FLAG_PER_PROBLEM   = 16
+    EVO_FLAG_PER_PROBLEM   = 16,
+    /* Debug switches for A/B comparisons of kernel forms (same results, other kernels); a
+     * production caller leaves them clear.  All other bits of `flags` must be zero. */
+    EVO_FLAG_DEBUG_NO_KV_RING   = 0x200,  /* dK/dV: the one-workgroup-per-problem kernel instead of the chunk-of-rows one */
+    EVO_FLAG_DEBUG_BIAS_TILES   = 0x800,  /* S <= 4: prepare the fp32 bias tiles instead of reading the caller's bias */
+    EVO_FLAG_DEBUG_NO_DQ_WIDE   = 0x1000, /* dQ: the kernels that split a row's keys over the waves, also without a dBias sum */
+    EVO_FLAG_DEBUG_NO_DQ_SPLIT  = 0x2000  /* dQ + dBias in one kernel, also where dQ and the dBias partials come from two */
 };
+#define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x200 | 0x800 | 0x1000 | 0x2000)
+
+/* A problem (b, s) whose every key carries a mask value below this is a "dead row"; see lse below. */
+#define EVOATTN_SHIFT_THRESHOLD (-1.0e5f)
 
 /* error codes */
 enum {
@@ -85,9 +95,10 @@ enum { EVO_PASS_FWD = 0, EVO_PASS_BWD = 1 };
  * (evoformer.py:648-650) is (S*N*H*D, S*N*D, N*D, D); a true per-head view of the same
  * tensor is (S*N*H*D, D, N*H*D, H*D).
  * lse is dense [B][H][S][N] fp32.  For a problem whose every key carries a mask value
- * below -1e4 the kernels subtract the largest mask value of the row from the scores
- * before the softmax (it cancels in O and in every gradient) and lse holds the
- * log-sum-exp of the shifted scores; otherwise lse = log sum_j exp(score_ij).
+ * below EVOATTN_SHIFT_THRESHOLD (-1e5) the scores are the mask values alone, less the
+ * largest of them (q.k and the bias are swamped by such a mask in fp32 arithmetic; the
+ * shift cancels in O and in every gradient), and lse holds the log-sum-exp of those
+ * shifted scores; otherwise lse = log sum_j exp(score_ij).
  */
 typedef struct EvoAttnParams {
     int32_t B, S, N, H, D;

@@ -21,6 +21,9 @@ the kept V rows; a single kept key returns that V row), softmax shift invariance
 permutation equivariance, an independent fp64 C restatement (oracle/evo_ref.c), a numpy
 fp64 index-by-index brute force, torch's scaled_dot_product_attention, gradcheck and
 central finite differences, and the zero-row-sum invariants of dS.
+backward_from_saved_output (the backward with delta taken from a saved, possibly rounded
+output) is pinned against autograd: with the unrounded fp64 output it must reproduce
+attention_fwd_bwd's gradients.
 """
 from __future__ import annotations
 
@@ -244,3 +247,67 @@ def bf16_ulp_bound(x: torch.Tensor) -> float:
     """Half a bf16 ulp at max|x|: the floor under any comparison of bf16 outputs."""
     m = float(x.abs().max())
     return 0.0 if m == 0 else 2.0 ** (math.floor(math.log2(m)) - 8)
+
+
+def backward_from_saved_output(Q, K, V, res_mask, pair_bias, dO, O_saved, layout="reference", s_chunk=None,
+                               compute_dtype=torch.float32, scaled_q_dtype=None, p_dtype=None):
+    """The backward as the reference's kernels arrange it, in compute_dtype on the given inputs:
+    delta = rowsum(dO * O) is formed from the output the forward SAVED (evoformer.py:313-323;
+    O_saved is that tensor, e.g. the forward's bf16 result) and dS = P * (dP - delta)
+    (evoformer.py:452-459, 600-611), instead of autograd's rowsum(P * dP) on the unrounded
+    probabilities.  With O_saved equal to the exact forward output this is autograd's result
+    (tests/test_oracle.py pins it that way); with the rounded output it shows what
+    the rounding of the saved activation alone does to the gradients.
+
+    Two more roundings of the reference's kernels can be switched on, each off by default:
+      scaled_q_dtype: the query operand is multiplied by the softmax scale and rounded to the
+        input dtype before the score matmul (evoformer.py:49, 433 scale Q in Q's dtype); here
+        the factor is scale * log2(e), the scores are brought back to natural units in fp32;
+      p_dtype: P and dS are cast to the input dtype before the gradient matmuls
+        (evoformer.py:459, 603, 611); dBias and dMask sum the unrounded dS (:456-458).
+
+    Returns dQ, dK, dV ([B,S,N,H,D]), dBias ([B,1,H,N,N]) and dMask ([B,S,1,1,N], floating mask only).
+    """
+    f = compute_dtype
+    Q, K, V, dO, O_saved = (t.to(f) for t in (Q, K, V, dO, O_saved))
+    res_mask, pair_bias = _cast(res_mask, f), _cast(pair_bias, f)
+    B, S, N, H, D = Q.shape
+    Qh, Kh, Vh, bias_h, mask_h = _head_views(Q, K, V, res_mask, pair_bias, layout)
+    dOh, Osh = to_heads(dO, layout), to_heads(O_saved, layout)
+    scale = 1.0 / (D ** 0.5)
+    log2e = 1.4426950408889634
+    step = S if not s_chunk else int(s_chunk)
+    dQh, dKh, dVh = torch.empty_like(Qh), torch.empty_like(Qh), torch.empty_like(Qh)
+    dbias = None if bias_h is None else torch.zeros_like(bias_h)
+    want_dmask = mask_h is not None and mask_h.dtype != torch.bool
+    dmask = torch.zeros((B, 1, S, 1, N), dtype=f, device=Q.device) if want_dmask else None
+    rnd = (lambda t: t) if p_dtype is None else (lambda t: t.to(p_dtype).to(f))
+    for s0 in range(0, S, step):
+        s1 = min(S, s0 + step)
+        q, k, v, g = Qh[:, :, s0:s1], Kh[:, :, s0:s1], Vh[:, :, s0:s1], dOh[:, :, s0:s1]
+        m = None if mask_h is None else mask_h[:, :, s0:s1]
+        if scaled_q_dtype is None:
+            scores = _scores_heads(q, k, bias_h, m)
+        else:
+            # _scores_heads multiplies by the scale itself: hand it the rounded operand divided by both factors
+            qs = (q * (scale * log2e)).to(scaled_q_dtype).to(f) / (scale * log2e)
+            scores = _scores_heads(qs, k, bias_h, m)
+        P = torch.softmax(scores, dim=-1)
+        dP = torch.matmul(g, v.transpose(3, 4))
+        delta = (g * Osh[:, :, s0:s1]).sum(-1, keepdim=True)
+        dS = P * (dP - delta)
+        if m is not None and m.dtype == torch.bool:
+            dS = dS.masked_fill(~m, 0.0)        # a replaced score passes no gradient (masked_fill, test.py:54)
+        dVh[:, :, s0:s1] = torch.matmul(rnd(P).transpose(3, 4), g)
+        dQh[:, :, s0:s1] = torch.matmul(rnd(dS), k) * scale
+        dKh[:, :, s0:s1] = torch.matmul(rnd(dS).transpose(3, 4), q) * scale
+        if dbias is not None:
+            dbias += dS.sum(2, keepdim=True)
+        if want_dmask:
+            dmask[:, :, s0:s1] = dS.sum((1, 3), keepdim=True)
+    out = {"dQ": from_heads(dQh, layout), "dK": from_heads(dKh, layout), "dV": from_heads(dVh, layout)}
+    if dbias is not None:
+        out["dBias"] = dbias.reshape(B, 1, H, N, N)
+    if dmask is not None:
+        out["dMask"] = dmask.reshape(B, S, 1, 1, N)
+    return out

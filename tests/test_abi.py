@@ -139,3 +139,42 @@ def test_error_strings(lib):
     with pytest.raises(_lib.EvoAttnError) as ei:
         _lib.check(_lib.EVO_EALIGN, "evoattn_fwd")
     assert ei.value.code == _lib.EVO_EALIGN and "evoattn_fwd" in str(ei.value)
+
+
+def header_flags():
+    text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
+    return {name: int(val, 0) for name, val in re.findall(r"\b(EVO_FLAG_[A-Z_]+)\s*=\s*(0x[0-9a-fA-F]+|\d+)", text)}
+
+
+def test_every_flag_bit_is_declared_in_the_header(lib):
+    """The binding's flag constants are the header's, every flag literal a test passes is one of them,
+    and a bit the header does not declare is rejected."""
+    declared = header_flags()
+    bound = {n: v for n, v in vars(_lib).items() if n.startswith("EVO_FLAG_")}
+    assert bound == declared
+    all_bits = 0
+    for v in declared.values():
+        assert v and v & (v - 1) == 0, "one bit per flag"
+        all_bits |= v
+    # no test spells a flag as a bare number
+    for fn in os.listdir(os.path.join(ROOT, "tests")):
+        if fn.endswith(".py") and fn != "test_abi.py":
+            src = open(os.path.join(ROOT, "tests", fn)).read()
+            assert not re.search(r"FLAGS\s*=\s*(0x[0-9a-fA-F]+|[1-9]\d*)\b", src), fn
+            assert not re.search(r"flags\s*=\s*(0x[0-9a-fA-F]+|[1-9]\d*)\b", src), fn
+    for bit in (0x20, 0x400, 0x4000, 1 << 30):
+        assert not bit & all_bits
+        p = good()
+        p.flags = bit
+        assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EINVAL
+    p = good()
+    p.flags = all_bits
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+
+
+def test_shift_threshold_is_the_header_constant():
+    text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
+    m = re.search(r"#define\s+EVOATTN_SHIFT_THRESHOLD\s+\((-[0-9.e]+)f\)", text)
+    assert m and float(m.group(1)) == -1.0e5
+    common = open(os.path.join(ROOT, "evoformer_triton_amd", "csrc", "common.h")).read()
+    assert "kShiftThreshold = EVOATTN_SHIFT_THRESHOLD" in common

@@ -20,10 +20,8 @@ from oracle import eager
 pytestmark = pytest.mark.gpu
 
 BF16_TOL = 2e-2
-FULL_REDUCED_ATOL = 2e-2   # absolute part of the bound on dBias at the full benchmark sizes
 # max-abs bound on O, dQ, dK, dV per benchmark configuration
 FULL_TOL = {"C2": BF16_TOL, "C3": BF16_TOL, "C4": BF16_TOL, "C5": BF16_TOL}
-FULL_DMASK_ATOL = 6e-2     # ... and on dMask, a sum over all heads and queries (2048..8192 terms)
 F32_TOL = 1e-5
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.npz")))
 
@@ -61,18 +59,29 @@ def max_err(a, b):
 REDUCED = ("dBias", "dMask")    # sums of dS over S rows / over heads and queries
 
 
-def assert_close(got, ref, tol, names=("O", "dQ", "dK", "dV", "dBias"), what="", ulp_names=REDUCED, ulps=1):
-    """max-abs <= tol on every tensor.  For the two reduced gradients, whose entries are
-    sums of many O(1) terms and reach |x| of 4..8 where one bf16 ulp is 3e-2..6e-2, the bound
-    for a 16-bit result is tol + one bf16 ulp of the reference entry (2^-7 relative)."""
+def half_ulp(x, dtype):
+    """Half a unit in the last place of a 16-bit format at each |x|, from the entry's own binade:
+    the most that rounding a result to that format moves it."""
+    bits = {torch.bfloat16: 8, torch.float16: 11}[dtype]          # significand bits, the implicit one included
+    floor = 2.0 ** (-126 if dtype == torch.bfloat16 else -14)
+    return torch.exp2(torch.floor(torch.log2(x.abs().clamp_min(floor))) - bits)
+
+
+def assert_close(got, ref, tol, names=("O", "dQ", "dK", "dV", "dBias"), what="", round_names=REDUCED):
+    """max-abs <= tol on every tensor.  For the tensors in `round_names` that come back in a
+    16-bit format the bound is, per element, tol plus half a unit in the last place of that
+    format at the entry (the larger of the two magnitudes decides the binade): the rounding of
+    the stored result itself, which no arithmetic can avoid.  By default these are the two reduced
+    gradients, whose entries are sums of many O(1) terms and reach |x| of 4..30."""
     errs, bad = {}, {}
     for n in names:
         if n not in ref or n not in got:
             continue
+        out_dtype = got[n].dtype
         a, b = got[n].detach().float().cpu(), ref[n].detach().float().cpu()
         errs[n] = (a - b).abs().max().item()
-        if n in ulp_names and tol > 1e-4:
-            ok = bool(((a - b).abs() <= tol + ulps * 2.0 ** -7 * b.abs()).all())
+        if n in round_names and out_dtype in (torch.bfloat16, torch.float16):
+            ok = bool(((a - b).abs() <= tol + half_ulp(torch.maximum(a.abs(), b.abs()), out_dtype)).all())
         else:
             ok = errs[n] <= tol
         if not ok:
@@ -325,13 +334,13 @@ def test_chunk_of_rows_kernels_match_per_problem_kernels(E, shape, mask):
                                            ((1, 4, 96, 2, 16), "q"), ((2, 2, 520, 1, 8), torch.float32)])
 def test_bias_read_from_the_callers_tensor_matches_the_prepared_tiles(E, shape, bias_dt):
     """With at most four S rows the kernels read the pair bias from the caller's tensor instead of
-    the prepared fp32 tiles (flag bit 0x800 keeps the tiles): the same fp32 product bias x log2(e)
+    the prepared fp32 tiles (EVO_FLAG_DEBUG_BIAS_TILES keeps the tiles): the same fp32 product bias x log2(e)
     enters the same MFMA, so the two forms agree to the last bit."""
     B, S, N, H, D = shape
     Q, K, V, m, bias, dO = make_case(B, S, N, H, D, "bool", bias_dt, torch.bfloat16, seed=9)
     from evoformer_triton_amd import _lib
     try:
-        E.FLAGS = 0x800 | _lib.EVO_FLAG_PER_PROBLEM      # the same one-workgroup-per-problem kernels, fed from tiles
+        E.FLAGS = _lib.EVO_FLAG_DEBUG_BIAS_TILES | _lib.EVO_FLAG_PER_PROBLEM      # the same one-workgroup-per-problem kernels, fed from tiles
         a = run_hip(E, Q, K, V, m, bias, dO)
     finally:
         E.FLAGS = 0
@@ -356,7 +365,8 @@ def test_dq_where_no_dbias_is_asked_for(E, case):
     """Without a pair bias, or with one that takes no gradient, dQ comes from the kernel whose
     waves own their query rows for all keys (`evoattn_kernels` names it); checked against the CPU
     oracle in fp32 and, to a 16-bit unit in the last place, against the kernels that split the keys
-    over the waves (flag bit 0x1000)."""
+    over the waves (EVO_FLAG_DEBUG_NO_DQ_WIDE)."""
+    from evoformer_triton_amd import _lib
     B, S, N, H, D, mask, bias_dt, dtype = case
     Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, bias_dt, dtype, seed=11)
     if m is not None and S > 2 and (m.dtype == torch.bool or dtype == torch.bfloat16):
@@ -375,7 +385,7 @@ def test_dq_where_no_dbias_is_asked_for(E, case):
         torch.cuda.synchronize()
         return {"O": o.detach(), "dQ": q.grad, "dK": k.grad, "dV": v.grad}
 
-    got, other = run(0), run(0x1000)
+    got, other = run(0), run(_lib.EVO_FLAG_DEBUG_NO_DQ_WIDE)
     assert_close(got, ref, BF16_TOL if dtype == torch.bfloat16 else 4e-3, ["O", "dQ", "dK", "dV"], what=str(case))
     ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
     for name in got:
@@ -393,7 +403,7 @@ def test_long_rows_sum_dbias_in_a_kernel_of_its_own(E, case):
     dim 32): dQ from
     the kernel whose waves own their query rows, the dBias partials from a second kernel that
     forms dS again (`evoattn_kernels` names both).  Against the CPU oracle in fp32, and against
-    the one kernel that does both (flag bit 0x2000) to a 16-bit unit in the last place."""
+    the one kernel that does both (EVO_FLAG_DEBUG_NO_DQ_SPLIT) to a 16-bit unit in the last place."""
     from evoformer_triton_amd import _lib
     B, S, N, H, D, mask, dtype = case
     Q, K, V, m, bias, dO = make_case(B, S, N, H, D, mask, "q", dtype, seed=17)
@@ -402,7 +412,7 @@ def test_long_rows_sum_dbias_in_a_kernel_of_its_own(E, case):
     ref = eager.attention_fwd_bwd(Q, K, V, m, bias, dO, compute_dtype=torch.float32)
     got = run_hip(E, Q, K, V, m, bias, dO)
     try:
-        E.FLAGS = 0x2000
+        E.FLAGS = _lib.EVO_FLAG_DEBUG_NO_DQ_SPLIT
         other = run_hip(E, Q, K, V, m, bias, dO)
     finally:
         E.FLAGS = 0
@@ -443,7 +453,7 @@ def test_dq_kernel_choice_is_reported(E):
     assert kernels((1, 64, 256, 4, 32), True, False) == "mfma_dq_wide"
     assert kernels((1, 64, 256, 4, 32), True, True) == "mfma_dq_ring"
     assert kernels((4, 1, 512, 8, 64), True, True) == "mfma_dq_wide"          # S = 1: dBias is dS
-    assert kernels((4, 1, 512, 8, 64), True, True, 0x1000) == "mfma_dq"
+    assert kernels((4, 1, 512, 8, 64), True, True, _lib.EVO_FLAG_DEBUG_NO_DQ_WIDE) == "mfma_dq"
     assert kernels((1, 2, 300, 1, 64), False, False) == "mfma_dq"             # six workgroups: keys split over waves
 
 
@@ -526,7 +536,7 @@ def test_head_dim_128_on_the_matrix_core(E, case):
     if b is not None and bias_grad:
         got["dBias"] = b.grad
         names.append("dBias")
-    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+    assert_close(got, ref, BF16_TOL, names, what=str(case), round_names=tuple(names))
     lib = _lib.load()
     lse = torch.empty((B, H, S, N), device=dev)
     mm, mk, mstr = E._prep_mask(on(m), B, S, N, q.device)
@@ -550,7 +560,7 @@ def test_head_dims_between_the_built_ones_are_padded(E, case):
     for n in ("O", "dQ", "dK", "dV"):
         assert got[n].shape == Q.shape and got[n].is_contiguous()
     assert_close(got, ref, BF16_TOL, ["O", "dQ", "dK", "dV", "dBias"] + (["dMask"] if fmask else []), what=str(case),
-                 ulp_names=("dQ", "dK", "dV", "dBias", "dMask"))
+                 round_names=("dQ", "dK", "dV", "dBias", "dMask"))
     # the registered operators take the same route
     dev = "cuda"
     o, lse, _, _ = torch.ops.evoattn.fwd(Q.to(dev), K.to(dev), V.to(dev), None if m is None else m.to(dev),
@@ -608,7 +618,7 @@ def test_rows_beyond_2048_keys(E, case):
     if b is not None and bias_grad:
         got["dBias"] = b.grad
         names.append("dBias")
-    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+    assert_close(got, ref, BF16_TOL, names, what=str(case), round_names=tuple(names))
     lib = _lib.load()
     mm, mk, mstr = E._prep_mask(on(m), B, S, N, q.device)
     bb, bdt, bstr = E._prep_bias(b, B, H, N, q.dtype, q.device)
@@ -686,7 +696,7 @@ def test_mask_edge_values(E, N):
         # probabilities rounded to bf16.  Eager evaluated in bf16 is 3.2e-2 away from the fp32
         # values on this input; the bound follows it.
         tol = BF16_TOL if N <= 96 else 3.5e-2
-        assert_close(got, ref, tol, what=f"mask {kind}", ulp_names=("dQ", "dK", "dV", "dBias"), ulps=2)
+        assert_close(got, ref, tol, what=f"mask {kind}", round_names=("dQ", "dK", "dV", "dBias"))
         Oh, Vh = eager.to_heads(got["O"].float().cpu()), eager.to_heads(V.float())
         assert (Oh[0, :, 2] - Vh[0, :, 2, 77:78]).abs().max() <= 1e-2       # single kept key: O = that V row
         assert (Oh[0, :, 1] - Vh[0, :, 1].mean(1, keepdim=True)).abs().max() <= 1e-2   # dead row: mean of V
@@ -727,7 +737,7 @@ def test_forward_maximum_found_in_a_later_key_block(E, where):
     # collect 256 products of probabilities rounded to bf16 (eager evaluated in bf16 is 0.19
     # away from the fp32 values on this input, the one-workgroup-per-problem kernels 0.025).
     tol = 3e-2 if where == "ramp" else BF16_TOL
-    assert_close(got, ref, tol, what=where, ulp_names=("dQ", "dK", "dV", "dBias"), ulps=2)
+    assert_close(got, ref, tol, what=where, round_names=("dQ", "dK", "dV", "dBias"))
 
 
 def test_checkpoint_recompute_and_no_grad(E):
@@ -936,7 +946,7 @@ def test_seeded_sweep_over_dispatch_boundaries(E, case):
     for n in names:
         assert torch.isfinite(got[n].float()).all(), f"{case}: {n} not finite"
     # tolerance plus one ulp of the 16-bit result (2^-7 relative covers bf16; fp16 is finer)
-    assert_close(got, ref, BF16_TOL, names, what=str(case), ulp_names=tuple(names), ulps=1)
+    assert_close(got, ref, BF16_TOL, names, what=str(case), round_names=tuple(names))
 
 
 # ------------------------------------------------------------------ full-size benchmark configurations
@@ -958,29 +968,43 @@ def test_benchmark_configs_full_size(E, cfg):
     e_self = {n: max_err(ref_bf16[n], ref_f32[n]) for n in main}
     mags = {n: ref_f32[n].abs().max().item() for n in main}
     print(f"\n{cfg}: max-abs vs eager-fp32 {e_f32} | vs eager-bf16 {e_bf} | eager-bf16 vs eager-fp32 {e_self} | max|ref| {mags}")
-    # (1) against the exact value of the eager formula on the same bf16 inputs (fp32 eager)
+    # (1) against the exact value of the eager formula on the same bf16 inputs (fp32 eager).
     # C5 (D=8, N=384) has |dK| up to 5.5 and |dQ| up to 3.3, where the rounding of the bf16
-    # result alone is 1.6e-2 / 0.8e-2: there the bound is the tolerance plus half a bf16
-    # ulp of the entry (the output rounding itself); eager in bf16 is 5.3e-2 away.
+    # result alone is up to 1.6e-2: there the bound is, per element, the tolerance plus half a
+    # bf16 unit in the last place of the entry (the output rounding itself); eager in bf16 is
+    # 5.3e-2 away.  The same shape in fp16 meets the plain 2e-2 (test_gpu_tolerance.py).
     assert_close(got, ref_f32, FULL_TOL[cfg], main, what=f"{cfg} vs eager fp32",
-                 ulp_names=("dQ", "dK", "dV") if cfg == "C5" else (), ulps=0.5)
+                 round_names=("dQ", "dK", "dV") if cfg == "C5" else ())
     # (2) against eager run as the reference writes it, all in bf16.  With a bf16 bias its
     # scores are themselves rounded to bf16 (test.py:53), so it sits up to e_self away from
     # the exact value; the HIP result must be within the tolerance of it once that is allowed.
     for n in main:
         assert e_bf[n] <= FULL_TOL[cfg] + e_self[n], f"{cfg} {n}: {e_bf[n]:.3e} vs eager bf16 (its own error {e_self[n]:.3e})"
-    # dBias (a sum of dS over S rows) and dMask (over heads and queries) reach |x| ~ 15..25
-    # here and come back in bf16, where one ulp is 6e-2..1.2e-1: an absolute 2e-2 cannot
-    # hold for them even for a correctly rounded result.  They are held to the reference's
-    # own relative criterion (rtol=1e-2, test.py:73-80) with atol = FULL_REDUCED_ATOL, against the exact value,
-    # and the absolute error is reported next to eager-bf16's own.
+    # (3) dBias (a sum of dS over S rows) and dMask (over heads and queries) reach |x| ~ 15..30
+    # here and come back in bf16, where half a unit in the last place is 3e-2..6e-2, and they
+    # inherit two roundings that the reference's kernels make as well: delta = <dO, O> is formed
+    # from the SAVED bf16 output (evoformer.py:313-323) and the query operand is multiplied by
+    # the scale in the input dtype (evoformer.py:49, 433; here from head dim 32 on, below the
+    # residue is carried).  The oracle restates the backward with exactly these two roundings
+    # (and P, dS cast before the gradient matmuls, evoformer.py:459, 603, 611); against that the
+    # kernels' own arithmetic is held to the tolerance plus the rounding of the stored result,
+    # per element, for every gradient; the distance of that restatement from fp32 eager is
+    # what the algorithm, not its implementation, costs, and is printed.
+    model = eager.backward_from_saved_output(xs["Q"], xs["K"], xs["V"], xs["mask"], xs["bias"], xs["dO"], got["O"],
+                                             s_chunk=chunk, scaled_q_dtype=torch.bfloat16 if D > 16 else None,
+                                             p_dtype=torch.bfloat16)
+    e_model = assert_close(got, model, FULL_TOL[cfg], ("dQ", "dK", "dV", "dBias", "dMask"), what=f"{cfg} vs the backward from the saved output",
+                           round_names=("dQ", "dK", "dV", "dBias", "dMask"))
+    alg = {n: max_err(model[n], ref_f32[n]) for n in ("dQ", "dK", "dV", "dBias", "dMask")}
     for n in ("dBias", "dMask"):
-        a, b = got[n].float(), ref_f32[n].float()
-        e_f32[n] = (a - b).abs().max().item()
+        e_f32[n] = max_err(got[n], ref_f32[n])
         e_self[n] = max_err(ref_bf16[n], ref_f32[n])
-        atol = FULL_REDUCED_ATOL if n == "dBias" else FULL_DMASK_ATOL
-        assert torch.allclose(a, b, atol=atol, rtol=1e-2), f"{n} max-abs {e_f32[n]:.3e} (|ref| max {b.abs().max().item():.2f})"
-    print(f"{cfg}: reduced gradients max-abs vs eager-fp32 { {n: e_f32[n] for n in ('dBias', 'dMask')} } | eager-bf16's own { {n: e_self[n] for n in ('dBias', 'dMask')} }")
+        # against fp32 eager itself: what the two shared roundings cost (measured just above) on top
+        a, b = got[n].float().cpu(), ref_f32[n].float().cpu()
+        bound = FULL_TOL[cfg] + alg[n] + half_ulp(torch.maximum(a.abs(), b.abs()), got[n].dtype)
+        assert bool(((a - b).abs() <= bound).all()), f"{cfg} {n}: max-abs {e_f32[n]:.3e} vs fp32 eager"
+    print(f"{cfg}: vs the backward from the saved output {e_model} | that restatement vs eager-fp32 {alg} | "
+          f"reduced gradients vs eager-fp32 { {n: e_f32[n] for n in ('dBias', 'dMask')} } | eager-bf16's own { {n: e_self[n] for n in ('dBias', 'dMask')} }")
 
 
 def test_full_size_properties_c2(E):

@@ -232,3 +232,45 @@ def test_flop_formula_and_inputs():
     assert torch.equal(x["bias"], y["bias"])
     z = eager.make_inputs("C2", shape=(1, 4, 64, 2, 32))
     assert z["mask"].shape == (1, 4, 1, 1, 64) and z["Q"].dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("mask_kind", ["add", "bool", None])
+@pytest.mark.parametrize("layout", ["reference", "ds4sci"])
+def test_backward_from_saved_output_is_autograd_when_the_output_is_unrounded(mask_kind, layout):
+    """The hand-arranged backward (delta from the saved output, dS = P (dP - delta)) against
+    autograd through the eager formula, both in fp64: equal when the saved output is the
+    exact one; and the rounding of the saved output moves dBias by what <dO, O - O_saved> predicts."""
+    x = eager.make_inputs("C2", shape=(2, 5, 48, 3, 16), dtype=torch.float64, seed=3)
+    m = x["mask"]
+    if mask_kind == "bool":
+        m = m == 0
+        m[0, 2] = False                      # a fully dropped row: no gradient through its scores
+    elif mask_kind is None:
+        m = None
+    ref = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], m, x["bias"], x["dO"], layout=layout)
+    got = eager.backward_from_saved_output(x["Q"], x["K"], x["V"], m, x["bias"], x["dO"], ref["O"], layout=layout,
+                                           s_chunk=2, compute_dtype=torch.float64)
+    for n, t in got.items():
+        assert (t - ref[n]).abs().max().item() < 1e-12, n
+    # the two optional roundings are identities when their format is the compute format ...
+    same = eager.backward_from_saved_output(x["Q"], x["K"], x["V"], m, x["bias"], x["dO"], ref["O"], layout=layout,
+                                            compute_dtype=torch.float64, scaled_q_dtype=torch.float64, p_dtype=torch.float64)
+    for n, t in same.items():
+        assert (t - ref[n]).abs().max().item() < 1e-12, n
+    # ... and move the gradients by no more than a 16-bit operand can (bf16: 2^-9 relative per element)
+    rough = eager.backward_from_saved_output(x["Q"], x["K"], x["V"], m, x["bias"], x["dO"], ref["O"], layout=layout,
+                                             compute_dtype=torch.float64, scaled_q_dtype=torch.bfloat16, p_dtype=torch.bfloat16)
+    for n, t in rough.items():
+        d = (t - ref[n]).abs().max().item()
+        assert 0 < d < 0.05 * ref[n].abs().max().item(), (n, d)
+    # a perturbed saved output: dS moves by -P * <dO, dO_saved>, so dBias by its sum over S
+    eps = 1e-3 * torch.randn_like(ref["O"])
+    pert = eager.backward_from_saved_output(x["Q"], x["K"], x["V"], m, x["bias"], x["dO"], ref["O"] + eps, layout=layout,
+                                            compute_dtype=torch.float64)
+    P = torch.softmax(eager._scores_heads(*eager._head_views(x["Q"], x["K"], x["V"], m, x["bias"], layout)[:2],
+                                          *eager._head_views(x["Q"], x["K"], x["V"], m, x["bias"], layout)[3:]), -1)
+    dd = (eager.to_heads(x["dO"], layout) * eager.to_heads(eps, layout)).sum(-1, keepdim=True)
+    pred = -(P * dd)
+    if mask_kind == "bool":
+        pred = pred.masked_fill(~m.reshape(2, 1, 5, 1, 48), 0.0)
+    assert ((pert["dBias"] - got["dBias"]).reshape(2, 3, 48, 48) - pred.sum(2)).abs().max().item() < 1e-12
