@@ -27,7 +27,8 @@ EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 
 EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_prep_bytes", "evoattn_bwd_workspace_bytes",
-           "evoattn_fwd", "evoattn_bwd", "evoattn_path", "evoattn_kernels")
+           "evoattn_fwd", "evoattn_fwd_static", "evoattn_bwd", "evoattn_path", "evoattn_kernels")
+EVOATTN_STATIC_PREP_BYTES = 16 << 20
 
 
 class EvoAttnParams(ctypes.Structure):
@@ -84,6 +85,8 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_bwd_workspace_bytes.argtypes = [P]
     lib.evoattn_fwd.restype = ctypes.c_int
     lib.evoattn_fwd.argtypes = [P, ctypes.c_void_p]
+    lib.evoattn_fwd_static.restype = ctypes.c_int
+    lib.evoattn_fwd_static.argtypes = [P, ctypes.c_void_p]
     lib.evoattn_bwd.restype = ctypes.c_int
     lib.evoattn_bwd.argtypes = [P, ctypes.c_void_p]
     lib.evoattn_path.restype = ctypes.c_char_p

@@ -6,6 +6,11 @@
 #include "common.h"
 #include "kernels.h"
 
+// Prepared operands of evoattn_fwd_static: one array per GPU the library runs on, held until the
+// process ends.  In host code the name stands for the symbol only; the array's device address is
+// asked for once per device (static_prep below) and only that address is handed to kernels.
+static __device__ __align__(256) unsigned char scratch[EVOATTN_STATIC_PREP_BYTES];
+
 namespace evo {
 
 static inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
@@ -357,6 +362,36 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream) {
     if (!mfma_ok(*p, EVO_PASS_FWD)) return launch_generic_fwd(*p, st);
     if ((rc = check_prep(*p))) return rc;
     return fwd_launches(*p, st);
+}
+
+// Device address of this GPU's copy of `scratch`, asked for on the first call on that device.
+static int static_prep(void **out) {
+    static std::atomic<void *> addr[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return EVO_EHIP - (int)hipGetLastError();
+    if (dev < 0 || dev >= 64) return EVO_EUNSUPPORTED;
+    void *ptr = addr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !ptr) return EVO_EHIP - (int)(err != hipSuccess ? err : hipErrorInvalidSymbol);
+        addr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return EVO_OK;
+}
+
+int evoattn_fwd_static(const EvoAttnParams *p, void *hip_stream) {
+    int rc = evoattn_check(p, EVO_PASS_FWD);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)hip_stream;
+    if (!mfma_ok(*p, EVO_PASS_FWD)) return launch_generic_fwd(*p, st);   // those kernels take no prepared operands
+    if (prep_layout(*p).total > (size_t)EVOATTN_STATIC_PREP_BYTES) return EVO_EWORKSPACE;
+    EvoAttnParams q = *p;
+    if ((rc = static_prep(&q.prep))) return rc;
+    q.prep_bytes = (size_t)EVOATTN_STATIC_PREP_BYTES;
+    // The prep kernel writes every byte of the array that this call's kernels read (bias tiles
+    // with their zero tile, mask rows, flags), so nothing of an earlier call has to be cleared.
+    return fwd_launches(q, st);
 }
 
 int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {

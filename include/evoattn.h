@@ -150,6 +150,20 @@ size_t evoattn_bwd_workspace_bytes(const EvoAttnParams *p);
 /* Enqueue the forward: writes o and lse. */
 int evoattn_fwd(const EvoAttnParams *p, void *hip_stream);
 
+/* evoattn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * forward allocates what it needs with torch (evoformer.py:654, 669-671).  Same kernels and results
+ * as evoattn_fwd, but the prepared operands live in an array inside the library instead of the
+ * caller's `prep` buffer: `prep` and `prep_bytes` of the parameter block are ignored, o and lse are
+ * still the caller's, and the call makes no hipMalloc / hipFree and no allocating library call.
+ * Limit: problems whose evoattn_prep_bytes() exceeds EVOATTN_STATIC_PREP_BYTES (16 MiB: rows up to
+ * about 512 keys with 8 heads, e.g. B=1 S=512 N=256 H=8 needs 8.3 MB) return EVO_EWORKSPACE.  The
+ * array is shared by every call on one GPU (each GPU has its own copy) and keeps the last call's
+ * contents: calls that overlap in time on one GPU race on it, so enqueue them on one stream or
+ * order them otherwise.  evoattn_bwd cannot reuse this prep (EVO_FLAG_PREP_VALID does not apply). */
+#define EVOATTN_STATIC_PREP_BYTES (16u << 20)
+int evoattn_fwd_static(const EvoAttnParams *p, void *hip_stream);
+
 /* Enqueue the backward: writes dq, dk, dv and, when non-NULL, dbias and dmask.
  * Deterministic: no floating-point atomics; two runs give bit-identical results. */
 int evoattn_bwd(const EvoAttnParams *p, void *hip_stream);

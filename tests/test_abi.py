@@ -178,3 +178,17 @@ def test_shift_threshold_is_the_header_constant():
     assert m and float(m.group(1)) == -1.0e5
     common = open(os.path.join(ROOT, "evoformer_triton_amd", "csrc", "common.h")).read()
     assert "kShiftThreshold = EVOATTN_SHIFT_THRESHOLD" in common
+
+
+def test_static_forward_rejects_oversized_problems_on_the_host(lib):
+    """evoattn_fwd_static checks the size of the prepared operands against its built-in array
+    before it touches the GPU."""
+    p = good(S=8, N=2048, H=8)
+    p.bias_dtype = _lib.EVO_BF16
+    assert lib.evoattn_prep_bytes(ctypes.byref(p)) > _lib.EVOATTN_STATIC_PREP_BYTES
+    assert lib.evoattn_fwd_static(ctypes.byref(p), None) == _lib.EVO_EWORKSPACE
+    p = good()
+    p.q = None
+    assert lib.evoattn_fwd_static(ctypes.byref(p), None) == _lib.EVO_EINVAL
+    text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
+    assert re.search(r"#define\s+EVOATTN_STATIC_PREP_BYTES\s+\(16u << 20\)", text)
