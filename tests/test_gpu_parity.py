@@ -90,6 +90,28 @@ def assert_close(got, ref, tol, names=("O", "dQ", "dK", "dV", "dBias"), what="",
     return errs
 
 
+def assert_close_to_modelled_backward(got, ref, inputs, tol, what):
+    """For inputs that put nearly all of a row's weight on a few keys, whose dK and dV then
+    collect hundreds of probabilities each rounded to 16 bits: the gradients are held to `tol`
+    (plus the rounding of the stored 16-bit result, per element) against the oracle's restatement
+    of the backward with the roundings the reference's kernels make too (delta from the saved
+    output, evoformer.py:313-323; the query operand scaled in the input dtype, :49, :433; P and
+    dS cast before the gradient matmuls, :459, :603, :611), and to tol plus that restatement's own
+    distance from fp32 eager against fp32 eager itself."""
+    Q, K, V, m, bias, dO = inputs
+    D = Q.shape[-1]
+    dt = Q.dtype
+    model = eager.backward_from_saved_output(Q, K, V, m, bias, dO, got["O"].cpu(), scaled_q_dtype=dt if D > 16 else None,
+                                             p_dtype=dt)
+    names = [n for n in ("dQ", "dK", "dV", "dBias") if n in got and n in model]
+    assert_close(got, model, tol, names, what=what + " vs the backward from the saved output", round_names=tuple(names))
+    for n in names:
+        a, b = got[n].detach().float().cpu(), ref[n].detach().float().cpu()
+        cost = (model[n].float() - b).abs().max().item()
+        bound = tol + cost + half_ulp(torch.maximum(a.abs(), b.abs()), got[n].dtype)
+        assert bool(((a - b).abs() <= bound).all()), f"{what} {n}: {(a - b).abs().max().item():.3e} vs fp32 eager (restatement {cost:.3e} away)"
+
+
 def load_case(path):
     z = np.load(path, allow_pickle=False)
     t = lambda k: torch.from_numpy(z[k]) if k in z.files else None
@@ -690,13 +712,13 @@ def test_mask_edge_values(E, N):
         got = run_hip(E, Q, K, V, m, bias, dO)
         for n, t in got.items():
             assert torch.isfinite(t.float()).all(), (kind, n)
-        # the single kept key collects dV = sum of all N dO rows, |dV| ~ 20..30: allow one
-        # bf16 ulp of the entry on top of the absolute bound
-        # At N = 256 five kept keys collect dK, dV from 256 queries each: sums of 256 products of
-        # probabilities rounded to bf16.  Eager evaluated in bf16 is 3.2e-2 away from the fp32
-        # values on this input; the bound follows it.
-        tol = BF16_TOL if N <= 96 else 3.5e-2
-        assert_close(got, ref, tol, what=f"mask {kind}", round_names=("dQ", "dK", "dV", "dBias"))
+        # The single kept key collects dV = sum of all N dO rows, |dV| ~ 20..30, and at N = 256
+        # five kept keys collect dK, dV from 256 queries each: sums of 256 products of
+        # probabilities rounded to bf16 (eager evaluated in bf16 is 3.2e-2 away from the fp32 values
+        # on this input).  O is held to the plain tolerance against fp32 eager, the gradients to
+        # the same tolerance against the restatement that makes the reference's roundings.
+        assert_close(got, ref, BF16_TOL, ("O",), what=f"mask {kind}")
+        assert_close_to_modelled_backward(got, ref, (Q, K, V, m, bias, dO), BF16_TOL, f"mask {kind}")
         Oh, Vh = eager.to_heads(got["O"].float().cpu()), eager.to_heads(V.float())
         assert (Oh[0, :, 2] - Vh[0, :, 2, 77:78]).abs().max() <= 1e-2       # single kept key: O = that V row
         assert (Oh[0, :, 1] - Vh[0, :, 1].mean(1, keepdim=True)).abs().max() <= 1e-2   # dead row: mean of V
@@ -735,9 +757,9 @@ def test_forward_maximum_found_in_a_later_key_block(E, where):
         assert torch.isfinite(t.float()).all(), (where, n)
     # The ramp puts nearly all of every row's weight on the last dozen keys, whose dK and dV
     # collect 256 products of probabilities rounded to bf16 (eager evaluated in bf16 is 0.19
-    # away from the fp32 values on this input, the one-workgroup-per-problem kernels 0.025).
-    tol = 3e-2 if where == "ramp" else BF16_TOL
-    assert_close(got, ref, tol, what=where, round_names=("dQ", "dK", "dV", "dBias"))
+    # away from the fp32 values on this input).
+    assert_close(got, ref, BF16_TOL, ("O",), what=where)
+    assert_close_to_modelled_backward(got, ref, (Q, K, V, m, bias, dO), BF16_TOL, where)
 
 
 def test_checkpoint_recompute_and_no_grad(E):
