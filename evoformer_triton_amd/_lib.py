@@ -19,7 +19,9 @@ EVO_FLAG_PREP_VALID = 2
 EVO_FLAG_ONLY_DQ = 4
 EVO_FLAG_ONLY_DKDV = 8
 EVO_FLAG_PER_PROBLEM = 16
+EVO_FLAG_DEBUG_OTHER_WIDTH = 0x100
 EVO_FLAG_DEBUG_NO_KV_RING = 0x200
+EVO_FLAG_DEBUG_FWD_BIAS_TILES = 0x400
 EVO_FLAG_DEBUG_BIAS_TILES = 0x800
 EVO_FLAG_DEBUG_NO_DQ_WIDE = 0x1000
 EVO_FLAG_DEBUG_NO_DQ_SPLIT = 0x2000
@@ -49,6 +51,7 @@ class EvoAttnParams(ctypes.Structure):
         ("dbias", ctypes.c_void_p), ("dmask", ctypes.c_void_p),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("prep", ctypes.c_void_p), ("prep_bytes", ctypes.c_size_t),
+        ("gate", ctypes.c_void_p), ("o_gated", ctypes.c_void_p), ("dgate", ctypes.c_void_p),
     ]
 
 

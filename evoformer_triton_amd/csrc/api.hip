@@ -28,6 +28,17 @@ static int check_common(const EvoAttnParams *p) {
     if (!p->q || !p->k || !p->v || !p->o || !p->lse) return EVO_EINVAL;
     if (!(p->scale == p->scale) || p->scale <= 0.0f) return EVO_EINVAL;
     if (p->flags & ~EVO_FLAG_ALL) return EVO_EINVAL;
+    if (p->gate) {
+        // the gate is read and its products written element for element like q: that needs a dense q-family
+        if (p->D % 8) return EVO_EUNSUPPORTED;
+        const int64_t st4[4] = {p->stride_b, p->stride_h, p->stride_s, p->stride_n};
+        const int64_t ext[4] = {p->B, p->H, p->S, p->N};
+        int64_t span = p->D;
+        for (int i = 0; i < 4; ++i) span += (ext[i] - 1) * st4[i];
+        if (span != (int64_t)p->B * p->H * p->S * p->N * p->D) return EVO_EUNSUPPORTED;
+    } else if (p->o_gated || p->dgate) {
+        return EVO_EINVAL;
+    }
     if (p->D != 8 && p->D != 16 && p->D != 32 && p->D != 64 && p->D != 128) return EVO_EUNSUPPORTED;
     if (p->stride_b < 0 || p->stride_h < 0 || p->stride_s < 0 || p->stride_n < p->D) return EVO_EINVAL;
     if (p->bias && (p->bias_stride_b < 0 || p->bias_stride_h < 0 || p->bias_stride_row < p->N)) return EVO_EINVAL;
@@ -41,6 +52,7 @@ static int check_common(const EvoAttnParams *p) {
     if (!aligned(p->q, es) || !aligned(p->k, es) || !aligned(p->v, es) || !aligned(p->o, es) || !aligned(p->lse, 4))
         return EVO_EALIGN;
     if (p->bias && !aligned(p->bias, elem_size(p->bias_dtype))) return EVO_EALIGN;
+    if (p->gate && (!aligned(p->gate, 16) || !aligned(p->o_gated, 16))) return EVO_EALIGN;   // rows are moved in 8- and 16-byte pieces (o_gated may be NULL in a backward call)
     if (p->mask_kind == EVO_MASK_F32 && !aligned(p->mask, 4)) return EVO_EALIGN;
     if ((p->mask_kind == EVO_MASK_BF16 || p->mask_kind == EVO_MASK_F16) && !aligned(p->mask, 2)) return EVO_EALIGN;
     return EVO_OK;
@@ -223,7 +235,7 @@ static int check_prep(const EvoAttnParams &p) {
 }
 
 struct WsLayout {
-    size_t delta, shift, dmask_part, dbias_part, total;
+    size_t delta, shift, dmask_part, dbias_part, dout_ungated, total;
     int n_chunks, chunk;
 };
 
@@ -237,6 +249,8 @@ static WsLayout ws_layout(const EvoAttnParams &p) {
     chunking(p, &w.n_chunks, &w.chunk);
     w.dbias_part = off;
     if (p.dbias && !dq_writes_dbias(p)) off += align_up((size_t)w.n_chunks * p.B * p.H * p.N * p.N * 4);
+    w.dout_ungated = off;
+    if (p.gate) off += align_up(rows * p.D * (size_t)elem_size(p.dtype));
     w.total = off;
     return w;
 }
@@ -250,6 +264,7 @@ static int check_bwd(const EvoAttnParams *p) {
         if (!aligned(p->dbias, elem_size(p->dbias_dtype))) return EVO_EALIGN;
     }
     if (p->dmask && !aligned(p->dmask, 4)) return EVO_EALIGN;
+    if (p->gate && (!p->dgate || !aligned(p->dgate, 16) || !aligned(p->dout, 16) || !aligned(p->o, 16))) return p->dgate ? EVO_EALIGN : EVO_EINVAL;
     const WsLayout w = ws_layout(*p);
     if (!p->workspace || p->workspace_bytes < w.total) return EVO_EWORKSPACE;
     if (!aligned(p->workspace, 256)) return EVO_EALIGN;
@@ -290,6 +305,7 @@ int evoattn_check(const EvoAttnParams *p, int pass) {
     if (rc) return rc;
     if (pass == EVO_PASS_BWD) return check_bwd(p);
     if (pass != EVO_PASS_FWD) return EVO_EINVAL;
+    if (p->gate && !p->o_gated) return EVO_EINVAL;   // the forward writes the gated output
     return EVO_OK;
 }
 
@@ -394,12 +410,22 @@ int evoattn_fwd_static(const EvoAttnParams *p, void *hip_stream) {
     return fwd_launches(q, st);
 }
 
-int evoattn_bwd(const EvoAttnParams *p, void *hip_stream) {
-    int rc = evoattn_check(p, EVO_PASS_BWD);
+int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
+    int rc = evoattn_check(p0, EVO_PASS_BWD);
     if (rc) return rc;
     hipStream_t st = (hipStream_t)hip_stream;
-    const WsLayout w = ws_layout(*p);
-    char *ws = (char *)p->workspace;
+    const WsLayout w = ws_layout(*p0);
+    char *ws = (char *)p0->workspace;
+    // With a gate, p0->dout is the gradient of the gated output: one pass over the rows forms the
+    // gradient of the ungated output (into the workspace) and of the gate, and the attention
+    // backward below runs on the former.
+    EvoAttnParams ungated = *p0;
+    if (p0->gate) {
+        if ((rc = launch_gate_bwd(*p0, ws + w.dout_ungated, st))) return rc;
+        ungated.dout = ws + w.dout_ungated;
+        ungated.gate = nullptr;
+    }
+    const EvoAttnParams *p = &ungated;
     Extra e{};
     e.n_chunks = w.n_chunks;
     e.chunk = w.chunk;

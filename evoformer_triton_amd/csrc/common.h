@@ -335,6 +335,25 @@ __device__ __forceinline__ void store4(T *dst, float a, float b, float c, float 
     *reinterpret_cast<typename Mfma<T>::v4 *>(dst) = v;
 }
 
+// sigmoid(x) = 1 / (1 + 2^(-x log2 e)): one exp2 and one reciprocal.
+__device__ __forceinline__ float sigmoidf(float x) { return __builtin_amdgcn_rcpf(1.0f + fast_exp2(-x * kLog2e)); }
+
+// The output gate on one accumulator tile's worth of a row: acc[r] *= sigmoid(gate[column of r]).
+// `grow` is this lane's row of the gate logits (laid out like the output row); a lane holds the
+// columns c0 + 8 (r / 4) + 4 g + r % 4, four consecutive ones per load.
+template <typename T>
+__device__ __forceinline__ void gate_row_tile(const T *grow, int c0, int ncols, f32x16 &acc, int g) {
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const int c = c0 + 8 * rr + 4 * g;
+        if (c < ncols) {
+            const typename Mfma<T>::v4 v = *reinterpret_cast<const typename Mfma<T>::v4 *>(grow + c);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[4 * rr + i] *= sigmoidf((float)v[i]);
+        }
+    }
+}
+
 // One accumulator tile's worth of a row to memory as T: lane (li, g) holds, for its row, the
 // 16 values of columns 8 (r / 4) + 4 g + r % 4; the two lanes of a row exchange halves so
 // that each stores 16 contiguous bytes (columns c0 + 16 p + 8 g .. + 7, p = 0, 1) instead of

@@ -62,6 +62,12 @@ __global__ void __launch_bounds__(64) gen_fwd(EvoAttnParams p) {
         T *O = (T *)p.o + pr.base + (int64_t)row * p.stride_n;
         float inv = 1.0f / l;
         for (int d = 0; d < D; ++d) O[d] = (T)(acc[d] * inv);
+        if (p.gate) {
+            const int64_t off = pr.base + (int64_t)row * p.stride_n;
+            const T *Gt = (const T *)p.gate + off;
+            T *Og = (T *)p.o_gated + off;
+            for (int d = 0; d < D; ++d) Og[d] = (T)(acc[d] * inv / (1.0f + expf(-(float)Gt[d])));
+        }
         p.lse[pr.row0 + row] = m + logf(l);
     }
 }
@@ -318,6 +324,54 @@ int launch_delta_generic(const EvoAttnParams &p, const Extra &e, hipStream_t st)
     }
     EVO_LAUNCH_CHECK();
     return EVO_OK;
+}
+
+// The gate's own backward, one pass over the rows: from the gradient of sigmoid(g) * O (in
+// p.dout), the gate logits g and the ungated O,
+//     dO = dout * sigmoid(g)                        -> dout_ungated (what the attention backward runs on)
+//     dg = dout * O * sigmoid(g) * (1 - sigmoid(g)) -> p.dgate
+// all three laid out like q.  One thread per 8 consecutive head-dim elements of one row.
+template <typename T>
+__global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_ungated) {
+    const int cpr = p.D / 8;   // 8-element pieces per row
+    const int64_t pieces = (int64_t)p.B * p.H * p.S * p.N * cpr;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= pieces) return;
+    const int c = (int)(i % cpr);
+    const int64_t r = i / cpr;
+    const Prob pr = decode_problem(p, (unsigned)(r / p.N));
+    const int64_t off = pr.base + (r % p.N) * p.stride_n + c * 8;
+    const T *go = (const T *)p.dout + off, *gl = (const T *)p.gate + off, *o = (const T *)p.o + off;
+    T *d_o = dout_ungated + off, *d_g = (T *)p.dgate + off;
+    // eight elements at a time: 16-byte loads and stores for the 16-bit types (the pieces are
+    // 16-byte aligned: dense tensors, head dim a multiple of 8), two of each for fp32
+    constexpr int V = sizeof(T) == 2 ? 8 : 4;
+    typedef T vec __attribute__((ext_vector_type(V)));
+#pragma unroll
+    for (int j0 = 0; j0 < 8; j0 += V) {
+        const vec a = *reinterpret_cast<const vec *>(go + j0), b = *reinterpret_cast<const vec *>(gl + j0),
+                  c2 = *reinterpret_cast<const vec *>(o + j0);
+        vec r_o, r_g;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const float sg = 1.0f / (1.0f + expf(-(float)b[j]));
+            const float gr = (float)a[j];
+            r_o[j] = (T)(gr * sg);
+            r_g[j] = (T)(gr * (float)c2[j] * sg * (1.0f - sg));
+        }
+        *reinterpret_cast<vec *>(d_o + j0) = r_o;
+        *reinterpret_cast<vec *>(d_g + j0) = r_g;
+    }
+}
+
+int launch_gate_bwd(const EvoAttnParams &p, void *dout_ungated, hipStream_t st) {
+    const int64_t pieces = (int64_t)p.B * p.H * p.S * p.N * (p.D / 8);
+    const unsigned grid = (unsigned)((pieces + 255) / 256);
+    if (p.dtype == EVO_F32) gate_bwd_kernel<float><<<grid, 256, 0, st>>>(p, (float *)dout_ungated);
+    else if (p.dtype == EVO_BF16) gate_bwd_kernel<bf16_t><<<grid, 256, 0, st>>>(p, (bf16_t *)dout_ungated);
+    else gate_bwd_kernel<f16_t><<<grid, 256, 0, st>>>(p, (f16_t *)dout_ungated);
+    hipError_t err = hipGetLastError();
+    return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }
 
 int launch_dmask_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st) {

@@ -650,11 +650,11 @@ static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 // N = 384, D = 32: 127 vs 149 us; N = 384, D = 8 within 3 %).
 template <typename T, int D>
 static int dkdv_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    // bit 0x100 of flags (not part of the public interface) inverts the choice, for comparison
+    // EVO_FLAG_DEBUG_OTHER_WIDTH inverts the choice, for comparison
     // ... unless there are too few problems for that: below four workgroups per CU (256 CUs) the
     // narrower form's twice as many workgroups fill the chip better
     const int64_t wgs = (int64_t)((p.N + 255) / 256) * p.B * p.H * p.S;
-    const bool wide = (p.N > 128 && wgs >= 1024) != ((p.flags & 0x100) != 0);
+    const bool wide = (p.N > 128 && wgs >= 1024) != ((p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) != 0);
     return wide ? dkdv_bias<T, D, 8>(p, e, st) : dkdv_bias<T, D, 4>(p, e, st);
 }
 

@@ -271,7 +271,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
 // flags (not part of the public interface) selects eight, for comparison.
 template <typename T, int D, bool HAS_BIAS, bool WRITE_DS>
 static int dqw_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    const int nw = (p.flags & 0x100) ? 8 : 4;
+    const int nw = (p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) ? 8 : 4;
     const unsigned grid = (unsigned)((p.N + nw * 32 - 1) / (nw * 32)) * (unsigned)(p.B * p.H * p.S);
     if (nw == 8) mfma_dq_wide<T, D, HAS_BIAS, 8, WRITE_DS><<<grid, 512, 0, st>>>(p, e);
     else mfma_dq_wide<T, D, HAS_BIAS, 4, WRITE_DS><<<grid, 256, 0, st>>>(p, e);

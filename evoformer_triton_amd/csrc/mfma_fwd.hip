@@ -254,6 +254,22 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
                         store4<T>(O + d0, oacc[dt][4 * rr] * inv, oacc[dt][4 * rr + 1] * inv,
                                   oacc[dt][4 * rr + 2] * inv, oacc[dt][4 * rr + 3] * inv);
                 }
+            if (p.gate) {   // uniform: sigmoid(gate) * O goes out as a second tensor, from the same registers
+                const int64_t off = pr.base + (int64_t)q * sn;
+                T *Og = (T *)p.o_gated + off;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= inv;
+                    gate_row_tile<T>((const T *)p.gate + off, dt * 32, D, oacc[dt], g);
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int d0 = dt * 32 + 8 * rr + 4 * g;
+                        if (d0 < D)
+                            store4<T>(Og + d0, oacc[dt][4 * rr], oacc[dt][4 * rr + 1], oacc[dt][4 * rr + 2], oacc[dt][4 * rr + 3]);
+                    }
+                }
+            }
         }
     }
 }
@@ -275,11 +291,10 @@ static int fwd_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     bool wide = p.N >= 256 && (rem == 0 || rem > 128);
     // ... and unless there are too few problems for that: below four workgroups per CU (256
     // CUs) the narrower form's twice as many workgroups fill the chip better (the reference's
-    // speed benchmark has 128 problems).  Bit 0x100 of flags (not part of the public
-    // interface) inverts the choice, for comparison.
+    // speed benchmark has 128 problems).  EVO_FLAG_DEBUG_OTHER_WIDTH inverts the choice, for comparison.
     const int64_t wgs = (int64_t)((p.N + 255) / 256) * p.B * p.H * p.S;
     if (wgs < 1024) wide = false;
-    if (p.flags & 0x100) wide = !wide;
+    if (p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) wide = !wide;
     return wide ? fwd_bias<T, D, 8>(p, e, st) : fwd_bias<T, D, 4>(p, e, st);
 }
 

@@ -465,6 +465,16 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 if (g == 0) p.lse[(int64_t)pid * p.N + q] = (m + __log2f(l)) * kLn2;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) store_row_tile<T>(O, dt * 32, D, oacc[dt], inv, g);
+                if (p.gate) {   // uniform: sigmoid(gate) * O goes out as a second tensor, from the same registers
+                    const int64_t off = base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) oacc[dt][r] *= inv;
+                        gate_row_tile<T>((const T *)p.gate + off, dt * 32, D, oacc[dt], g);
+                        store_row_tile<T>((T *)p.o_gated + off, dt * 32, D, oacc[dt], 1.0f, g);
+                    }
+                }
             }
         }
 #pragma unroll
@@ -498,11 +508,11 @@ template <typename T>
 static int fwdr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     if (p.bias_dtype == EVO_NONE) return fwdr_launch<T, EVO_D, 0>(p, e, st);
     // The 16-bit form reads the caller's bias rows in 16-byte pieces; where it applies it is the
-    // faster one (64 resident registers instead of 128, no spills).  Bit 0x400 of flags (not
-    // part of the public interface) selects the other form, for comparison.
+    // faster one (64 resident registers instead of 128, no spills).  EVO_FLAG_DEBUG_FWD_BIAS_TILES selects
+    // the other form, for comparison.
     const bool rows16 = p.bias_dtype == p.dtype && p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 &&
                         p.bias_stride_b % 8 == 0 && p.bias_stride_h % 8 == 0 && p.bias_stride_row % 8 == 0;
-    return (rows16 && !(p.flags & 0x400)) ? fwdr_launch<T, EVO_D, 2>(p, e, st) : fwdr_launch<T, EVO_D, 1>(p, e, st);
+    return (rows16 && !(p.flags & EVO_FLAG_DEBUG_FWD_BIAS_TILES)) ? fwdr_launch<T, EVO_D, 2>(p, e, st) : fwdr_launch<T, EVO_D, 1>(p, e, st);
 }
 
 // Largest N this kernel takes for the head dim (0: not built for it).

@@ -141,6 +141,12 @@ def _check_qkv(Q, K, V):
         raise RuntimeError("EvoformerAttention runs on the GPU only (no CPU implementation); move Q, K, V to one cuda device")
 
 
+def _check_gate(gate, Q):
+    if gate.shape != Q.shape or gate.dtype != Q.dtype or gate.device != Q.device:
+        raise ValueError(f"gate must have the shape, dtype and device of Q: {tuple(Q.shape)} {Q.dtype}, got {tuple(gate.shape)} {gate.dtype}")
+    return gate.contiguous()
+
+
 def _prep_bytes_upper(lib, p):
     """Size of the prep buffer that holds for any alignment of the bias: with few S rows the
     library reads an aligned bias in place and needs less; an odd address asks for the most."""
@@ -152,7 +158,7 @@ def _prep_bytes_upper(lib, p):
     return n
 
 
-def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
+def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False, gate=None):
     """Validate, allocate O / LSE / prep with torch and enqueue the forward on the current
     stream.  Returns what the backward needs: the tensors as the kernels saw them."""
     _check_qkv(Q, K, V)
@@ -176,9 +182,18 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False):
         nbytes = _prep_bytes_upper(lib, p) if prep_upper else lib.evoattn_prep_bytes(ctypes.byref(p))
         prep = _alloc_bytes(nbytes, Q.device)
         p.prep, p.prep_bytes = _ptr(prep), prep.numel()
+        Og = None
+        if gate is not None:                                   # sigmoid(gate) * O from the forward's epilogue
+            Gp = _padded(_check_gate(gate, Qc), Dp)
+            Og = torch.empty_like(Qp)
+            p.gate, p.o_gated = _ptr(Gp), _ptr(Og)
         _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(Q.device)), "evoattn_fwd")
         if Dp != D:
             O = O[..., :D].contiguous()
+            Og = None if Og is None else Og[..., :D].contiguous()
+    if gate is not None:
+        return Qc, Kc, Vc, mask, bias, O, lse, prep, (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype)), \
+            (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype)), Og
     mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
     return Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta
@@ -199,7 +214,7 @@ def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
 
 
 def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_meta, need_dmask, need_dbias,
-              prep_valid=True):
+              prep_valid=True, gate=None):
     """Allocate the gradients and the workspace and enqueue the backward; `mask` and `bias`
     are the tensors the forward's kernels saw.  Returns (dQ, dK, dV, dmask, dbias) with the
     last two in the shape and dtype of the caller's tensors, or None."""
@@ -220,6 +235,7 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
     Dp = _pad_head_dim(D)
     if Dp != D:                                                  # zero columns, as in the forward
         Q, K, V, O, dO = (_padded(t, Dp) for t in (Q, K, V, O, dO))
+        gate = None if gate is None else _padded(gate, Dp)
     want_dbias = bool(need_dbias and bias is not None)
     want_dmask = bool(need_dmask and mask is not None and mask.is_floating_point())
     with torch.cuda.device(Q.device):
@@ -234,6 +250,10 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
         if want_dmask:
             dmask = torch.empty((B, S, N), device=Q.device, dtype=torch.float32)
             p.dmask = _ptr(dmask)
+        dgate = None
+        if gate is not None:                                     # dO here is the gradient of the gated output
+            dgate = torch.empty_like(Q)
+            p.gate, p.dgate = _ptr(gate), _ptr(dgate)
         ws = _alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), Q.device)
         p.workspace, p.workspace_bytes = _ptr(ws), ws.numel()
         if not prep_valid:                                       # not the forward's tensors: prepare again
@@ -258,6 +278,8 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
         if shape[1] == 1 and S > 1:
             dmask = dmask.sum(1, keepdim=True)
         dmask = dmask.to(dtype)
+    if gate is not None:
+        return dQ, dK, dV, dmask, dbias, (dgate[..., :D].contiguous() if Dp != D else dgate)
     return dQ, dK, dV, dmask, dbias
 
 
@@ -399,11 +421,40 @@ class _PerHeadAttention(torch.autograd.Function):
         return _backward(ctx, dO, ctx.needs_input_grad[3], ctx.needs_input_grad[4])
 
 
-def evoformer_attention(Q, K, V, res_mask=None, pair_bias=None, layout: str = "reference"):
-    """Functional form; layout "reference" (flat reshape) or "ds4sci" (per-head permute)."""
+class _GatedAttention(torch.autograd.Function):
+    """sigmoid(gate) * attention(Q, K, V, res_mask, pair_bias) with the gate applied in the forward
+    kernel's epilogue (the step that follows the attention in an Evoformer block; the reference
+    returns O ungated, evoformer.py:735).  `gate`: the gate logits, shaped like Q.  The ungated O is
+    kept for the backward, which returns the gate's gradient as a sixth value."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, res_mask, pair_bias, gate, layout):
+        Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta, Og = _fwd_impl(Q, K, V, res_mask, pair_bias, layout,
+                                                                                 gate=gate)
+        ctx.save_for_backward(Qc, Kc, Vc, mask, bias, O, lse, prep, gate.contiguous())
+        ctx.layout, ctx.mask_meta, ctx.bias_meta = layout, mask_meta, bias_meta
+        return Og
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dOg):
+        Q, K, V, mask, bias, O, lse, prep, gate = ctx.saved_tensors
+        dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Q, K, V, mask, bias, O, lse, prep, ctx.layout, ctx.mask_meta,
+                                                    ctx.bias_meta, ctx.needs_input_grad[3], ctx.needs_input_grad[4], gate=gate)
+        return dQ, dK, dV, dmask, dbias, dgate, None
+
+
+def evoformer_attention(Q, K, V, res_mask=None, pair_bias=None, layout: str = "reference", gate=None):
+    """Functional form; layout "reference" (flat reshape) or "ds4sci" (per-head permute).
+    With `gate` (logits shaped like Q) the result is sigmoid(gate) * O, formed in the forward
+    kernel's epilogue."""
     fn = EvoformerAttention if layout == "reference" else _PerHeadAttention
     if layout not in ("reference", "ds4sci"):
         raise ValueError(f"unknown layout {layout!r}")
+    if gate is not None:
+        if Q.numel() == 0:
+            return torch.sigmoid(gate) * fn.apply(Q, K, V, res_mask, pair_bias)
+        return _GatedAttention.apply(Q, K, V, res_mask, pair_bias, gate, layout)
     return fn.apply(Q, K, V, res_mask, pair_bias)
 
 

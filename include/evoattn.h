@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define EVOATTN_VERSION 1
+#define EVOATTN_VERSION 2   /* 2: gate, o_gated, dgate appended to EvoAttnParams */
 
 /* element types */
 enum {
@@ -65,12 +65,14 @@ enum {
     EVO_FLAG_PER_PROBLEM   = 16,
     /* Debug switches for A/B comparisons of kernel forms (same results, other kernels); a
      * production caller leaves them clear.  All other bits of `flags` must be zero. */
-    EVO_FLAG_DEBUG_NO_KV_RING   = 0x200,  /* dK/dV: the one-workgroup-per-problem kernel instead of the chunk-of-rows one */
+    EVO_FLAG_DEBUG_OTHER_WIDTH  = 0x100,  /* one-workgroup-per-problem kernels: the other of their two workgroup widths (4 / 8 waves) */
+    EVO_FLAG_DEBUG_NO_KV_RING   = 0x200,
+    EVO_FLAG_DEBUG_FWD_BIAS_TILES = 0x400, /* chunk-of-rows forward: fp32 bias tiles as C operands instead of the caller's 16-bit rows */  /* dK/dV: the one-workgroup-per-problem kernel instead of the chunk-of-rows one */
     EVO_FLAG_DEBUG_BIAS_TILES   = 0x800,  /* S <= 4: prepare the fp32 bias tiles instead of reading the caller's bias */
     EVO_FLAG_DEBUG_NO_DQ_WIDE   = 0x1000, /* dQ: the kernels that split a row's keys over the waves, also without a dBias sum */
     EVO_FLAG_DEBUG_NO_DQ_SPLIT  = 0x2000  /* dQ + dBias in one kernel, also where dQ and the dBias partials come from two */
 };
-#define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x200 | 0x800 | 0x1000 | 0x2000)
+#define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x100 | 0x200 | 0x400 | 0x800 | 0x1000 | 0x2000)
 
 /* A problem (b, s) whose every key carries a mask value below this is a "dead row"; see lse below. */
 #define EVOATTN_SHIFT_THRESHOLD (-1.0e5f)
@@ -133,6 +135,20 @@ typedef struct EvoAttnParams {
      * buffer to evoattn_bwd with EVO_FLAG_PREP_VALID to skip the second derivation. */
     void       *prep;
     size_t      prep_bytes;
+
+    /* Output gate of the Evoformer block, fused (all three NULL: no gate).  `gate` holds the gate
+     * logits g, element for element like q (same dtype, same four strides).  evoattn_fwd then
+     * writes sigmoid(g) * O to o_gated (laid out like o) from its epilogue, in addition to the
+     * ungated O in `o`, which stays the tensor the backward takes delta = <dO, O> from.
+     * evoattn_bwd takes in `dout` the gradient of o_gated, forms dO = dout * sigmoid(g) and
+     * dgate = dout * O * sigmoid(g) * (1 - sigmoid(g)) in one pass over the rows (dgate laid out
+     * like q; dO goes to the workspace, which grows by one tensor of q's size) and runs the
+     * attention backward on that dO.  The q-family must be dense (its four strides a permutation
+     * of a contiguous [B][S][N][H][D] or [B][H][S][N][D] tensor).  The reference returns O
+     * ungated (evoformer.py:735); its callers apply the gate as a separate step. */
+    const void *gate;
+    void       *o_gated;
+    void       *dgate;
 } EvoAttnParams;
 
 int         evoattn_version(void);

@@ -126,7 +126,7 @@ def attention(Q, K, V, res_mask=None, pair_bias=None, layout="reference",
 
 def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
                       compute_dtype: Optional[torch.dtype] = None,
-                      s_chunk: Optional[int] = None) -> Dict[str, torch.Tensor]:
+                      s_chunk: Optional[int] = None, gate=None) -> Dict[str, torch.Tensor]:
     """Forward + autograd backward of the eager formula (test.py:47-62).
 
     Returns O, dQ, dK, dV, LSE and, when present, dBias ([B,1,H,N,N]) and dMask (only for
@@ -136,6 +136,11 @@ def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
     s_chunk: evaluate s_chunk rows of the head-major S axis at a time and accumulate
     dBias across chunks.  Rows are independent apart from that sum, so the result is the
     same formula with [B,H,s_chunk,N,N] of scores alive instead of [B,H,S,N,N].
+
+    gate: gate logits shaped like Q.  The block's output is then sigmoid(gate) * O (the step
+    that follows the attention in an Evoformer block; the reference returns O ungated,
+    evoformer.py:735, and leaves the gate to its caller); dO is the gradient of that gated
+    output, "Og" holds it, "O" the ungated attention output, "dGate" the gradient of the logits.
     """
     Q, K, V, dO = (_cast(t, compute_dtype).detach() for t in (Q, K, V, dO))
     res_mask = _cast(res_mask, compute_dtype)
@@ -145,6 +150,9 @@ def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
     dOh = to_heads(dO, layout)
     want_dmask = mask_h is not None and mask_h.dtype != torch.bool
     step = S if not s_chunk else int(s_chunk)
+    Gh = None if gate is None else to_heads(_cast(gate, compute_dtype).detach(), layout)
+    Ogh = None if gate is None else torch.empty_like(Qh)
+    dGh = None if gate is None else torch.empty_like(Qh)
 
     Oh = torch.empty_like(Qh)
     dQh, dKh, dVh = torch.empty_like(Qh), torch.empty_like(Qh), torch.empty_like(Qh)
@@ -168,7 +176,14 @@ def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
                 m = m.requires_grad_()
                 leaves.append(m)
         o, l = _attention_heads(q, k, v, b, m)
-        grads = torch.autograd.grad(o, leaves, dOh[:, :, s0:s1])
+        if Gh is None:
+            grads = torch.autograd.grad(o, leaves, dOh[:, :, s0:s1])
+        else:
+            gl = Gh[:, :, s0:s1].detach().requires_grad_()
+            og = torch.sigmoid(gl) * o
+            grads = torch.autograd.grad(og, leaves + [gl], dOh[:, :, s0:s1])
+            Ogh[:, :, s0:s1] = og.detach()
+            dGh[:, :, s0:s1] = grads[-1]
         Oh[:, :, s0:s1] = o.detach()
         lse[:, :, s0:s1] = l.detach()
         dQh[:, :, s0:s1], dKh[:, :, s0:s1], dVh[:, :, s0:s1] = grads[0], grads[1], grads[2]
@@ -186,6 +201,8 @@ def attention_fwd_bwd(Q, K, V, res_mask, pair_bias, dO, layout="reference",
         out["dBias"] = dbias.reshape(B, 1, H, N, N)
     if dmask is not None:
         out["dMask"] = dmask.reshape(B, S, 1, 1, N)
+    if Gh is not None:
+        out["Og"], out["dGate"] = from_heads(Ogh, layout), from_heads(dGh, layout)
     return out
 
 

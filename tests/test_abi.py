@@ -28,12 +28,12 @@ def test_every_declared_symbol_is_exported(lib):
     assert set(names) == set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.evoattn_version() == 1
+    assert lib.evoattn_version() == 2
 
 
 def test_struct_layout_matches_header():
     # 12 x 4-byte fields, 9 x int64, 14 pointers, one size_t, then prep pointer + size; no padding
-    assert ctypes.sizeof(EvoAttnParams) == 12 * 4 + 9 * 8 + 14 * 8 + 8 + 16
+    assert ctypes.sizeof(EvoAttnParams) == 12 * 4 + 9 * 8 + 14 * 8 + 8 + 16 + 3 * 8        # ... and the three gate pointers
     assert EvoAttnParams.stride_b.offset == 48 and EvoAttnParams.q.offset == 120
 
 
@@ -162,7 +162,7 @@ def test_every_flag_bit_is_declared_in_the_header(lib):
             src = open(os.path.join(ROOT, "tests", fn)).read()
             assert not re.search(r"FLAGS\s*=\s*(0x[0-9a-fA-F]+|[1-9]\d*)\b", src), fn
             assert not re.search(r"flags\s*=\s*(0x[0-9a-fA-F]+|[1-9]\d*)\b", src), fn
-    for bit in (0x20, 0x400, 0x4000, 1 << 30):
+    for bit in (0x20, 0x40, 0x4000, 1 << 30):
         assert not bit & all_bits
         p = good()
         p.flags = bit

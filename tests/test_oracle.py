@@ -274,3 +274,36 @@ def test_backward_from_saved_output_is_autograd_when_the_output_is_unrounded(mas
     if mask_kind == "bool":
         pred = pred.masked_fill(~m.reshape(2, 1, 5, 1, 48), 0.0)
     assert ((pert["dBias"] - got["dBias"]).reshape(2, 3, 48, 48) - pred.sum(2)).abs().max().item() < 1e-12
+
+
+def test_gate_closed_forms_and_gradcheck():
+    """The gated output sigmoid(g) * O: a large gate is the identity (and passes no gradient to the
+    gate), g = 0 halves the output and gives dGate = dO * O / 4, and the whole map passes
+    gradcheck in fp64 together with the attention's own inputs."""
+    x = eager.make_inputs("C2", shape=(1, 3, 12, 2, 8), dtype=torch.float64, seed=9)
+    plain = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"])
+    big = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], gate=torch.full_like(x["Q"], 50.0))
+    for n in ("dQ", "dK", "dV", "dBias", "dMask"):
+        assert (big[n] - plain[n]).abs().max().item() < 1e-12, n
+    assert (big["Og"] - plain["O"]).abs().max().item() < 1e-12 and big["dGate"].abs().max().item() < 1e-12
+    half = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], gate=torch.zeros_like(x["Q"]))
+    assert (half["Og"] - 0.5 * plain["O"]).abs().max().item() < 1e-15
+    assert (half["dGate"] - 0.25 * x["dO"] * plain["O"]).abs().max().item() < 1e-15
+    for n in ("dQ", "dK", "dV", "dBias"):                       # dO reaches the attention halved
+        assert (half[n] - 0.5 * plain[n]).abs().max().item() < 1e-12, n
+    # chunked evaluation and the per-head layout agree with the plain evaluation
+    g = torch.randn(x["Q"].shape, dtype=torch.float64, generator=torch.Generator().manual_seed(1))
+    a = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], gate=g)
+    b = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], gate=g, s_chunk=2)
+    for n in a:
+        assert (a[n] - b[n]).abs().max().item() < 1e-12, n
+
+    def f(q, k, v, bias, gl):
+        o = eager.attention(q, k, v, x["mask"], bias, layout="ds4sci")
+        return torch.sigmoid(gl) * o
+
+    leaves = [t.clone().requires_grad_() for t in (x["Q"], x["K"], x["V"], x["bias"], g)]
+    assert torch.autograd.gradcheck(f, leaves, eps=1e-6, atol=1e-6)
+    c = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], gate=g, layout="ds4sci")
+    grads = torch.autograd.grad(f(*leaves), leaves, x["dO"])
+    assert (c["dGate"] - grads[4]).abs().max().item() < 1e-12 and (c["dQ"] - grads[0]).abs().max().item() < 1e-12
