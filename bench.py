@@ -31,14 +31,21 @@ if ROOT not in sys.path:
 
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch (reads + writes) from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the counter reads for a plain 256 MiB copy (2.000 and 1.000); the commands
-# and raw readings are kept with the other profile summaries.  Not measurable from
-# inside this script, so only the profiled workload has a figure.
-MEASURED_HBM_BYTES_PER_LAUNCH = {
-    ("C2", "mfma_fwd_ring"): 295.4e6, ("C2", "mfma_dq_ring"): 446.9e6, ("C2", "mfma_dkdv_ring"): 450.4e6,
-    ("C2-nobias", "mfma_fwd_ring"): 289.6e6, ("C2-nobias", "mfma_dq_wide"): 419.5e6, ("C2-nobias", "mfma_dkdv_ring"): 430.3e6,
-}
+# HBM bytes per launch (reads + writes) come from two `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE),
+# each scaled by what the counter reads for a plain 256 MiB copy.  They cannot be measured from
+# inside this script: profiles/traffic.json holds them per workload and kernel together with the
+# commit they were measured at (the summaries next to it give the commands and raw readings).
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(config, kernel):
+    """(bytes per launch, commit of the measurement) for the dominant kernel of a profiled workload, else (None, None)."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            t = json.load(f)
+        return t["bytes_per_launch"][config][kernel.split("+")[-1]], t["commit"]
+    except (OSError, KeyError, ValueError):
+        return None, None
 
 
 def parse():
@@ -309,6 +316,7 @@ def main():
                    "bwd_dq": 6 * t_b + 2 * l_b + 2 * b_b,       # Q,K,V,dO,O,LSE -> dQ, delta, dBias
                    "bwd_dkdv": 6 * t_b + 2 * l_b + b_b}         # Q,K,V,dO,LSE,delta -> dK,dV
     hbm_gbs = phase_bytes[dom] / t_phase[dom] / 1e9
+    traffic, traffic_commit = measured_traffic(args.config, kernel_names[dom].split(" ")[0]) if bias is not None else (None, None)
     out = {
         "metric": "fwd+bwd TFLOP/s (S=%d N=%d H=%d D=%d)" % (S, N, H, D),
         "value": f_full / dt / 1e12,
@@ -333,10 +341,12 @@ def main():
         "c_abi_tflops": f_full / t_abi / 1e12,
         "kernel_ms": {kernel_names[n]: t * 1e3 for n, t in t_phase.items()},
         "peak_mem_bytes_beyond_inputs": int(peak_extra),
+        "kernel_ms_note": "each phase is timed between two HIP events inside a step (forward, dQ, dK/dV in that order), so the "
+                          "three figures include the gaps between the launches and can sum to more than ms_per_step, which is "
+                          "wall time over back-to-back steps",
         "roofline": {"bound": "mfma", "kernel": kernel_names[dom], "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS,
-                     "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get((args.config + ("" if bias is not None else "-nobias"),
-                                                                    kernel_names[dom].split("+")[-1])),
+                     "traffic": traffic, "traffic_measured_at_commit": traffic_commit,
                      "flops_per_launch": phases[dom][1], "avg_launch_ms": t_phase[dom] * 1e3,
                      # the same launch against the other ceiling: by intensity (flops / bytes below
                      # peak flops / peak bytes) the memory ceiling is the lower of the two here
