@@ -654,7 +654,12 @@ static int dkdv_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     // ... unless there are too few problems for that: below four workgroups per CU (256 CUs) the
     // narrower form's twice as many workgroups fill the chip better
     const int64_t wgs = (int64_t)((p.N + 255) / 256) * p.B * p.H * p.S;
-    const bool wide = (p.N > 128 && wgs >= 1024) != ((p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) != 0);
+    // ... and unless the last 256-key workgroup of a problem would be at most half full at a small head dim, where
+    // staging Q and dO a second time is cheap (bf16, S = 1024, H = 8, N = 384: 444 vs 531 us at head dim 8, 535 vs
+    // 571 us at 16; N = 320, head dim 8: 171 vs 222 us; at head dim 32 the two forms are level, 124 vs 123 us)
+    const int rem = p.N % 256;
+    const bool half_empty = D <= 16 && rem > 0 && rem <= 128;
+    const bool wide = (p.N > 128 && wgs >= 1024 && !half_empty) != ((p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) != 0);
     return wide ? dkdv_bias<T, D, 8>(p, e, st) : dkdv_bias<T, D, 4>(p, e, st);
 }
 
