@@ -425,7 +425,8 @@ class _GatedAttention(torch.autograd.Function):
     """sigmoid(gate) * attention(Q, K, V, res_mask, pair_bias) with the gate applied in the forward
     kernel's epilogue (the step that follows the attention in an Evoformer block; the reference
     returns O ungated, evoformer.py:735).  `gate`: the gate logits, shaped like Q.  The ungated O is
-    kept for the backward, which returns the gate's gradient as a sixth value."""
+    kept for the backward, which returns the gate's gradient as a sixth value.  Eager calls only: the
+    operators registered for torch.compile (torch.ops.evoattn.fwd / .bwd) are the ungated ones."""
 
     @staticmethod
     def forward(ctx, Q, K, V, res_mask, pair_bias, gate, layout):

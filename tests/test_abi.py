@@ -192,3 +192,35 @@ def test_static_forward_rejects_oversized_problems_on_the_host(lib):
     assert lib.evoattn_fwd_static(ctypes.byref(p), None) == _lib.EVO_EINVAL
     text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
     assert re.search(r"#define\s+EVOATTN_STATIC_PREP_BYTES\s+\(16u << 20\)", text)
+
+
+def test_gate_validation_on_the_host(lib):
+    """The gate's pointers are checked before any launch: the forward needs o_gated, the backward
+    dgate and one more tensor of workspace, and the q-family has to be dense."""
+    p = good()
+    fake = 0x10000
+    p.gate = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EINVAL        # no o_gated
+    p.o_gated = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL        # no dgate
+    p.dgate = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == 0
+    q = good()
+    need_plain = lib.evoattn_bwd_workspace_bytes(ctypes.byref(q))
+    assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) >= need_plain + 1 * 4 * 64 * 2 * 32 * 2   # + dO, bf16
+    p.gate = 0x10008
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EALIGN
+    p.gate = fake
+    p.stride_s *= 2                                                                         # rows with gaps: not dense
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EUNSUPPORTED
+    # the per-head layout of the same dense tensor is fine
+    p = good()
+    B, S, N, H, D = 1, 4, 64, 2, 32
+    p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * H * D, D, N * H * D, H * D
+    p.gate = p.o_gated = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    # gate outputs without a gate are a mistake
+    p = good()
+    p.dgate = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL
