@@ -224,3 +224,20 @@ def test_gate_validation_on_the_host(lib):
     p = good()
     p.dgate = fake
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL
+
+
+def test_header_is_plain_c_and_the_library_loads_from_c(tmp_path):
+    """tests/abi_check.c, compiled as strict C99 against include/evoattn.h, loads the library with
+    dlopen and exercises the host-side validation: the boundary holds without Python or torch."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    exe = tmp_path / "abi_check"
+    src = os.path.join(ROOT, "tests", "abi_check.c")
+    subprocess.check_call([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-D_POSIX_C_SOURCE=200809L",
+                           "-I", os.path.join(ROOT, "include"), src, "-o", str(exe), "-ldl"])
+    out = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    assert f"sizeof(EvoAttnParams) = {ctypes.sizeof(EvoAttnParams)}" in out.stdout
