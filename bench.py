@@ -43,7 +43,8 @@ def measured_traffic(config, kernel):
     try:
         with open(TRAFFIC_JSON) as f:
             t = json.load(f)
-        return t["bytes_per_launch"][config][kernel.split("+")[-1]], t["commit"]
+        names = [k for k in kernel.split("+") if k != "prep_kernel"]           # a phase of two kernels: both launches
+        return sum(t["bytes_per_launch"][config][k] for k in names), t["commit"]
     except (OSError, KeyError, ValueError):
         return None, None
 
