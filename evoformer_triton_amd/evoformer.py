@@ -388,6 +388,72 @@ def _op_backward(ctx, dO, dlse, dprep, dseen):
 _op_fwd.register_autograd(_op_backward, setup_context=_op_setup_context)
 
 
+# ---- the gated pair (sigmoid(gate) * O from the forward's epilogue, the gate's gradient from the backward) ----
+
+@torch.library.custom_op("evoattn::fwd_gated", mutates_args=(), device_types="cuda")
+def _op_fwd_gated(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
+                  pair_bias: Optional[torch.Tensor], gate: torch.Tensor, per_head: bool
+                  ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(O_gated, O, LSE, prep bytes, seen): `evoattn::fwd` with the output gate applied in the epilogue;
+    the ungated O is returned as well because the backward takes delta from it."""
+    out = _fwd_impl(Q, K, V, res_mask, pair_bias, "ds4sci" if per_head else "reference", prep_upper=True, gate=gate)
+    return out[10], out[5], out[6], out[7], _seen(out[3], out[4])
+
+
+@_op_fwd_gated.register_fake
+def _(Q, K, V, res_mask, pair_bias, gate, per_head):
+    o, lse, prep, seen = torch.ops.evoattn.fwd(Q, K, V, res_mask, pair_bias, per_head)
+    return Q.new_empty(Q.shape), o, lse, prep, seen
+
+
+@torch.library.custom_op("evoattn::bwd_gated", mutates_args=(), device_types="cuda")
+def _op_bwd_gated(dOg: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
+                  pair_bias: Optional[torch.Tensor], gate: torch.Tensor, O: torch.Tensor, lse: torch.Tensor,
+                  prep: torch.Tensor, seen: torch.Tensor, per_head: bool, need_dbias: bool, need_dmask: bool
+                  ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dQ, dK, dV, dMask, dBias, dGate) from the gradient of the gated output."""
+    B, S, N, H, D = Q.shape
+    Qc, Kc, Vc = Q.contiguous(), K.contiguous(), V.contiguous()
+    mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
+    bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
+    mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
+    bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+    same = bool(torch.equal(seen.cpu(), _seen(mask, bias)))
+    dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Qc, Kc, Vc, mask, bias, O.contiguous(), lse, prep,
+                                                "ds4sci" if per_head else "reference", mask_meta, bias_meta,
+                                                need_dmask, need_dbias, prep_valid=same, gate=_check_gate(gate, Qc))
+    none = Q.new_empty((0,))
+    return dQ, dK, dV, (none if dmask is None else dmask), (none.clone() if dbias is None else dbias), dgate
+
+
+@_op_bwd_gated.register_fake
+def _(dOg, Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen, per_head, need_dbias, need_dmask):
+    want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
+    want_dbias = need_dbias and pair_bias is not None
+    return (Q.new_empty(Q.shape), Q.new_empty(Q.shape), Q.new_empty(Q.shape),
+            res_mask.new_empty(res_mask.shape) if want_dmask else Q.new_empty((0,)),
+            pair_bias.new_empty(pair_bias.shape) if want_dbias else Q.new_empty((0,)), Q.new_empty(Q.shape))
+
+
+def _op_gated_setup_context(ctx, inputs, output):
+    Q, K, V, res_mask, pair_bias, gate, per_head = inputs
+    Og, O, lse, prep, seen = output
+    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen)
+    ctx.per_head = per_head
+
+
+def _op_gated_backward(ctx, dOg, dO_unused, dlse, dprep, dseen):
+    Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen = ctx.saved_tensors
+    need_dmask = bool(ctx.needs_input_grad[3] and res_mask is not None and res_mask.is_floating_point())
+    need_dbias = bool(ctx.needs_input_grad[4] and pair_bias is not None)
+    dQ, dK, dV, dmask, dbias, dgate = torch.ops.evoattn.bwd_gated(dOg, Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen,
+                                                                  ctx.per_head, need_dbias, need_dmask)
+    return dQ, dK, dV, (dmask if need_dmask else None), (dbias if need_dbias else None), dgate, None
+
+
+_op_fwd_gated.register_autograd(_op_gated_backward, setup_context=_op_gated_setup_context)
+
+
 class EvoformerAttention(torch.autograd.Function):
     """`EvoformerAttention.apply(Q, K, V, res_mask, pair_bias)` (evoformer.py:633-862).
 
@@ -425,20 +491,33 @@ class _GatedAttention(torch.autograd.Function):
     """sigmoid(gate) * attention(Q, K, V, res_mask, pair_bias) with the gate applied in the forward
     kernel's epilogue (the step that follows the attention in an Evoformer block; the reference
     returns O ungated, evoformer.py:735).  `gate`: the gate logits, shaped like Q.  The ungated O is
-    kept for the backward, which returns the gate's gradient as a sixth value.  Eager calls only: the
-    operators registered for torch.compile (torch.ops.evoattn.fwd / .bwd) are the ungated ones."""
+    kept for the backward, which returns the gate's gradient as a sixth value.  Under torch.compile the
+    same work goes through torch.ops.evoattn.fwd_gated / .bwd_gated."""
 
     @staticmethod
     def forward(ctx, Q, K, V, res_mask, pair_bias, gate, layout):
+        if torch.compiler.is_compiling():
+            # under torch.compile the device work is the registered operator (opaque to the tracer)
+            Og, O, lse, prep, seen = torch.ops.evoattn.fwd_gated(Q, K, V, res_mask, pair_bias, gate, layout == "ds4sci")
+            ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen)
+            ctx.layout, ctx.through_ops = layout, True
+            return Og
         Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta, Og = _fwd_impl(Q, K, V, res_mask, pair_bias, layout,
                                                                                  gate=gate)
         ctx.save_for_backward(Qc, Kc, Vc, mask, bias, O, lse, prep, gate.contiguous())
-        ctx.layout, ctx.mask_meta, ctx.bias_meta = layout, mask_meta, bias_meta
+        ctx.layout, ctx.mask_meta, ctx.bias_meta, ctx.through_ops = layout, mask_meta, bias_meta, False
         return Og
 
     @staticmethod
     @torch.autograd.function.once_differentiable
     def backward(ctx, dOg):
+        if ctx.through_ops:
+            Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen = ctx.saved_tensors
+            need_dmask, need_dbias = bool(ctx.needs_input_grad[3]), bool(ctx.needs_input_grad[4])
+            dQ, dK, dV, dmask, dbias, dgate = torch.ops.evoattn.bwd_gated(dOg, Q, K, V, res_mask, pair_bias, gate, O, lse, prep,
+                                                                          seen, ctx.layout == "ds4sci", need_dbias, need_dmask)
+            want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
+            return dQ, dK, dV, (dmask if want_dmask else None), (dbias if need_dbias and pair_bias is not None else None), dgate, None
         Q, K, V, mask, bias, O, lse, prep, gate = ctx.saved_tensors
         dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Q, K, V, mask, bias, O, lse, prep, ctx.layout, ctx.mask_meta,
                                                     ctx.bias_meta, ctx.needs_input_grad[3], ctx.needs_input_grad[4], gate=gate)

@@ -119,3 +119,41 @@ def test_gated_attention_at_the_headline_size(E):
     a, b = got["dBias"].float(), ref["dBias"].float()
     half_ulp = torch.exp2(torch.floor(torch.log2(torch.maximum(a.abs(), b.abs()).clamp_min(2.0 ** -126))) - 8)
     assert bool(((a - b).abs() <= 2e-2 + half_ulp).all()), (a - b).abs().max().item()
+
+
+def test_gated_attention_compiles_without_a_graph_break(E):
+    """The gated Function inside a compiled block (fullgraph=True, aot_eager backend) goes through
+    torch.ops.evoattn.fwd_gated / .bwd_gated and returns what the eager block returns; the two
+    operators pass torch.library's schema and fake-tensor checks."""
+    shape = (1, 4, 128, 2, 32)
+    x = eager.make_inputs("C2", shape=shape, seed=12)
+    gate = torch.randn(shape, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    dev = torch.device("cuda", torch.cuda.current_device())
+
+    def block(q, k, v, mask, bias, g):
+        return E.evoformer_attention(q, k, v, mask, bias * 1.0, gate=g * 1.0) + 1.0
+
+    def run(fn):
+        q, k, v = (x[n].to(dev).requires_grad_() for n in "QKV")
+        b, g = x["bias"].to(dev).requires_grad_(), gate.to(dev).requires_grad_()
+        out = fn(q, k, v, x["mask"].to(dev), b, g)
+        out.backward(x["dO"].to(dev))
+        torch.cuda.synchronize()
+        return [out.detach(), q.grad, k.grad, v.grad, b.grad, g.grad]
+
+    want = run(block)
+    torch._dynamo.reset()
+    compiled = torch.compile(block, backend="aot_eager", fullgraph=True)
+    for _ in range(2):
+        got = run(compiled)
+        for a, w in zip(got, want):
+            assert a.shape == w.shape and a.dtype == w.dtype
+            assert (a.float() - w.float()).abs().max().item() <= 1e-6 + 2.0 ** -7 * w.float().abs().max().item()
+    q, k, v = (x[n].to(dev).requires_grad_() for n in "QKV")
+    b, g, m = x["bias"].to(dev).requires_grad_(), gate.to(dev).requires_grad_(), x["mask"].to(dev)
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration")
+    torch.library.opcheck(torch.ops.evoattn.fwd_gated, (q, k, v, m, b, g, False), test_utils=tests)
+    with torch.no_grad():
+        og, o, lse, prep, seen = torch.ops.evoattn.fwd_gated(q, k, v, m, b, g, False)
+    torch.library.opcheck(torch.ops.evoattn.bwd_gated, (x["dO"].to(dev), q.detach(), k.detach(), v.detach(), m, b.detach(), g.detach(),
+                                                        o, lse, prep, seen, False, True, False), test_utils=tests[:2])
