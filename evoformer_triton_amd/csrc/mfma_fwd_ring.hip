@@ -8,9 +8,9 @@
 //   * a workgroup has 8 waves = 256 query rows (all of them) and a fixed head; wave w keeps
 //     the bias of (query tile w) x (all keys) for the whole chunk of S rows, as it sits in
 //     memory: 16-bit values, 64 registers, read once per chunk straight from the caller's
-//     tensor.  It enters the scores through the matrix core, S^T += (I c) B^T with I the
-//     identity and c = log2(e) as hi + lo of the 16-bit type (4 MFMAs per 32 x 32 tile on a
-//     unit that is mostly idle; exact to 2^-17);
+//     tensor.  It enters the scores through the matrix core, S^T = I B^T with I the identity
+//     (2 MFMAs per 32 x 32 tile, exact), and is brought to log2 units by one fp32
+//     multiplication per score;
 //   * K, V and the mask columns of row s+1 are requested (16 bytes per lane and load) before
 //     row s is computed out of one LDS buffer and written into the other one afterwards; a
 //     wave's own Q rows are prefetched straight into its registers;
