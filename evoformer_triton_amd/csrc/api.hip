@@ -190,7 +190,7 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
 }
 
 struct PrepLayout {
-    size_t bq, bk, bt, m2, m2a, dead, total;
+    size_t bq, bk, bq16, bk16, bt, m2, m2a, dead, total;
     int bias_batches;
 };
 
@@ -203,6 +203,13 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
     size_t off = 0;
     w.bq = off; off += align_up(tiles);
     w.bk = off; off += align_up(tiles);
+    // the same tiles in 16 bits for a bias in the dtype of q
+    const bool t16_ok = tiles != 0 && p.bias_dtype == p.dtype && p.dtype != EVO_F32;
+    w.bq16 = w.bk16 = (size_t)-1;
+    if (t16_ok) {
+        w.bq16 = off; off += align_up(tiles / 2);
+        w.bk16 = off; off += align_up(tiles / 2);
+    }
     // transposed 16-bit copy for the kernels that keep bias columns resident
     const bool bt_ok = p.bias && !bias_direct(p) && p.bias_dtype == p.dtype && p.N % 8 == 0;
     w.bt = bt_ok ? off : (size_t)-1;
@@ -221,6 +228,8 @@ static void fill_prep(const EvoAttnParams &p, Extra &e) {
     e.bias_direct = bias_direct(p) ? 1 : 0;
     e.bq = (float *)(base + w.bq);
     e.bk = (float *)(base + w.bk);
+    e.bq16 = w.bq16 == (size_t)-1 ? nullptr : (unsigned short *)(base + w.bq16);
+    e.bk16 = w.bk16 == (size_t)-1 ? nullptr : (unsigned short *)(base + w.bk16);
     e.bt = w.bt == (size_t)-1 ? nullptr : (void *)(base + w.bt);
     e.m2 = (uint2 *)(base + w.m2);
     e.m2a = (uint4 *)(base + w.m2a);

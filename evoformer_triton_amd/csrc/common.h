@@ -45,13 +45,15 @@ struct Extra {
     // prepared operands of the matrix-core kernels (written by the prep kernel)
     float *bq;         // bias * log2(e) in accumulator-tile order, lane = query  [Bb][H][NT][NT][64][16]
     float *bk;         // same, lane = key
+    unsigned short *bq16;  // a bias in the dtype of q as given (16 bits, not scaled) in the same tile order, lane = query; else null
+    unsigned short *bk16;  // same, lane = key
     uint2 *m2;         // additive mask * log2(e), shifted, clamped, as (hi, mid, lo, 0) of T  [B][S][NT*32]
     uint4 *m2a;        // the same mask rows as ready-made 16-byte operand chunks (hi, mid, lo, 1, 1, 1, 0, 0),
                        // padded with the floor to a multiple of 256 keys                        [B][S][NP256]
     void *bt;          // the bias transposed (key-major), in the dtype of q; null unless the bias has
                        // that dtype and N is a multiple of 8                                    [Bb][H][N][N]
     int *dead;         // [B][S] 1 where every key of the row is masked out
-    int64_t zero_tile; // offset (floats) of an all-zero tile inside bq and bk
+    int64_t zero_tile; // offset (elements) of an all-zero tile inside bq, bk, bq16 and bk16
     long long *trace;  // trace builds only: 16 timestamps per wave
 };
 
@@ -243,6 +245,27 @@ __device__ __forceinline__ void unpack2<f16_t>(unsigned w, float &lo, float &hi)
     const h2 v = __builtin_bit_cast(h2, w);
     lo = (float)v[0];
     hi = (float)v[1];
+}
+
+// A 32x32 bias tile as prepared in 16 bits: this lane's 16 accumulator entries, two to a
+// register (entry 2 i in the low half of word i).  `unpack_tile16` gives them as fp32 times `mul`.
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+struct Tile16 {
+    u32x4_t w[2];
+};
+__device__ __forceinline__ void load_tile16(const unsigned short *lane_tile, Tile16 &t) {
+    t.w[0] = *reinterpret_cast<const u32x4_t *>(lane_tile);
+    t.w[1] = *reinterpret_cast<const u32x4_t *>(lane_tile + 8);
+}
+template <typename T>
+__device__ __forceinline__ void unpack_tile16(const Tile16 &t, float mul, f32x16 &dst) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float lo, hi;
+        unpack2<T>(t.w[i >> 2][i & 3], lo, hi);
+        dst[2 * i] = lo * mul;
+        dst[2 * i + 1] = hi * mul;
+    }
 }
 
 // A 32x32 bias tile in accumulator order, times `mul`, straight from the caller's tensor (for

@@ -22,6 +22,8 @@
 // additions of the fp32 dS, as the reference adds fp32 dS at :456-459), writes one partial
 // per chunk, and a second kernel adds the partials in a fixed order: no floating-point
 // atomics, bit-reproducible.
+#include <type_traits>
+
 #include "bwd_common.h"
 #include "kernels.h"
 
@@ -331,14 +333,20 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 #define EVO_TK(slot) do {} while (0)
 #endif
 
-template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
+// BT: 0 no bias; 1 fp32 tiles (times log2 e) or, for very few S rows, the caller's columns; 2 the
+// tiles of a bias in the dtype of q as given (half the bytes per tile, 8 registers in flight
+// instead of 16; unpacked and multiplied by log2 e right before they are used)
+template <typename T, int D, int BT, int NW, int ROWS>
 __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_dkdv(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef KvGeo<D> R;
+    constexpr bool HAS_BIAS = BT != 0, TILE16 = BT == 2;
+    typedef typename std::conditional<TILE16, Tile16, f32x16>::type CTile;   // a bias tile on its way
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
     constexpr int NTH = NW * 64;
     constexpr int BK = NW * 32;
-    constexpr bool PREFETCH = NW == 4;       // the 8-wave form runs at 128 registers: prefetching there spills (227 vs 187 us)
+    // the 8-wave form runs at 128 registers: prefetching a 16-register tile there spills (227 vs 187 us)
+    constexpr bool PREFETCH = NW == 4 || TILE16;
     constexpr int BQS = ROWS, C = R::C;      // query rows staged per round
     constexpr int TPS = BQS / 32;            // query tiles per stage
     typedef typename Mfma<T>::v8 v8;
@@ -394,8 +402,22 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     const bool bf32 = p.bias_dtype == EVO_F32;
     const char *bmat = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h) * (bf32 ? 4 : 2);
     const float bmul = dead ? 0.0f : kLog2e;
-    auto load_btile = [&](int qt, f32x16 &dst) {
-        if (HAS_BIAS && bdirect) {   // uniform
+    const unsigned short *btile16 = !TILE16 ? nullptr
+                                    : dead  ? e.bk16 + e.zero_tile + lane * 16
+                                            : e.bk16 + (((int64_t)bb * p.H + pr.h) * NT * NT + ktc) * 1024 + lane * 16;
+    auto cval = [&](const CTile &t) -> f32x16 {
+        if constexpr (TILE16) {
+            f32x16 v;
+            unpack_tile16<T>(t, bmul, v);
+            return v;
+        } else {
+            return t;
+        }
+    };
+    auto load_btile = [&](int qt, CTile &dst) {
+        if constexpr (TILE16) {
+            load_tile16(btile16 + (int64_t)min(qt, NT - 1) * bstep, dst);
+        } else if (HAS_BIAS && bdirect) {   // uniform
             if (bf32) bias_tile_cols<T, true>(bmat, keyc, min(qt, NT - 1) * 32, p.N, (unsigned)p.bias_stride_row, g, bmul, dst);
             else bias_tile_cols<T, false>(bmat, keyc, min(qt, NT - 1) * 32, p.N, (unsigned)p.bias_stride_row, g, bmul, dst);
         } else if (HAS_BIAS) {
@@ -461,7 +483,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     };
 
     // one 32-query tile against this wave's 32 keys
-    auto compute = [&](int qtile, f32x16 &ctile) {
+    auto compute = [&](int qtile, CTile &ctile) {
         const int qb = (qtile % TPS) * 32;
         f32x16 acc, dp;
 #pragma unroll
@@ -480,7 +502,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
             }
             if (ks == 0) {
                 if (HAS_BIAS) {
-                    acc = Mfma<T>::mma(qa, kf[0], ctile);
+                    acc = Mfma<T>::mma(qa, kf[0], cval(ctile));
                 } else {
                     f32x16 z;
 #pragma unroll
@@ -557,7 +579,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
         }
     };
 
-    f32x16 ctile;
+    CTile ctile;
     if (PREFETCH) load_btile(0, ctile);
     stage(0);
     // K with the mask columns, V with ones against -delta
@@ -623,11 +645,11 @@ static int dq_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.bias_dtype == EVO_NONE ? dq_ntw<T, D, false>(p, e, st) : dq_ntw<T, D, true>(p, e, st);
 }
 
-template <typename T, int D, bool HAS_BIAS, int NW, int ROWS>
+template <typename T, int D, int BT, int NW, int ROWS>
 static int dkdv_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned grid = (unsigned)((p.N + NW * 32 - 1) / (NW * 32)) * (unsigned)(p.B * p.H * p.S);
     constexpr int lds = KvGeo<D>::lds_bytes(ROWS);   // at most 56 KB up to head dim 64, 100 KB at 128
-    auto kern = mfma_dkdv<T, D, HAS_BIAS, NW, ROWS>;
+    auto kern = mfma_dkdv<T, D, BT, NW, ROWS>;
     if constexpr (lds > 64 * 1024) {
         static PerDevice done{};
         if (const int rc = ensure_dynamic_lds((const void *)kern, lds, done, nullptr)) return rc;
@@ -639,10 +661,12 @@ static int dkdv_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 template <typename T, int D, int NW>
 static int dkdv_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     typedef KvGeo<D> R;
+    const int bt = p.bias_dtype == EVO_NONE ? 0 : (e.bk16 && !e.bias_direct) ? 2 : 1;
     if (NW == 4 && p.N <= 128)
-        return p.bias_dtype == EVO_NONE ? dkdv_launch<T, D, false, NW, 128>(p, e, st) : dkdv_launch<T, D, true, NW, 128>(p, e, st);
-    return p.bias_dtype == EVO_NONE ? dkdv_launch<T, D, false, NW, R::BQS>(p, e, st)
-                                    : dkdv_launch<T, D, true, NW, R::BQS>(p, e, st);
+        return bt == 0 ? dkdv_launch<T, D, 0, NW, 128>(p, e, st)
+             : bt == 2 ? dkdv_launch<T, D, 2, NW, 128>(p, e, st) : dkdv_launch<T, D, 1, NW, 128>(p, e, st);
+    return bt == 0 ? dkdv_launch<T, D, 0, NW, R::BQS>(p, e, st)
+         : bt == 2 ? dkdv_launch<T, D, 2, NW, R::BQS>(p, e, st) : dkdv_launch<T, D, 1, NW, R::BQS>(p, e, st);
 }
 
 // 8 waves (256 keys) per workgroup stage Q and dO once for twice the keys: measured faster

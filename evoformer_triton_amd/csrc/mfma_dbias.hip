@@ -68,10 +68,8 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
     const v8 vaug = aug8<T>(one3, zero3);
 
     // bias tiles (this wave's query tile x the block's key tiles) in accumulator order, as the
-    // 16-bit values of the caller's tensor, two to a register: the prepared fp32 tile holds
-    // fl(b * log2(e)); times ln 2 and rounded to 16 bits that is b again (the product is off by a
-    // few units of 2^-24, half a 16-bit unit is 2^-9 or 2^-12 of b).  Per use they are unpacked
-    // and multiplied by log2(e) in fp32, the product the prepared tile holds.
+    // 16-bit values of the caller's tensor, two to a register (the prepared 16-bit tiles).  Per
+    // use they are unpacked and multiplied by log2(e) in fp32, the product the fp32 tiles hold.
     const int bb = e.bias_batches > 1 ? b : 0;
     const int qtc = min(q0 >> 5, NT - 1);
     unsigned bres[TPW][8];
@@ -79,17 +77,10 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
 #pragma unroll
     for (int j = 0; j < TPW; ++j) {
         const int kt = min(k0 / 32 + j, NT - 1);
-        const float *src = e.bq + ((((int64_t)bb * p.H + h) * NT + qtc) * NT + kt) * 1024 + lane * 16;
+        Tile16 t;
+        load_tile16(e.bq16 + ((((int64_t)bb * p.H + h) * NT + qtc) * NT + kt) * 1024 + lane * 16, t);
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-            const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
-            typename Mfma<T>::v4 t;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) t[i] = (T)(v[i] * kLn2);
-            const uint2 w = __builtin_bit_cast(uint2, t);
-            bres[j][2 * rr] = w.x;
-            bres[j][2 * rr + 1] = w.y;
-        }
+        for (int i = 0; i < 8; ++i) bres[j][i] = t.w[i >> 2][i & 3];
 #pragma unroll
         for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
     }

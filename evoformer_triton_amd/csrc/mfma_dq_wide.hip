@@ -38,8 +38,12 @@ struct DqWideGeo {
 
 typedef short s16x4w __attribute__((ext_vector_type(4)));
 
-template <typename T, int D, bool HAS_BIAS, int NW, bool WRITE_DS>
+// BT: 0 no bias; 1 fp32 tiles (times log2 e) or, for very few S rows, the caller's rows; 2 the
+// tiles of a bias in the dtype of q as given (half the bytes per tile; unpacked and multiplied by
+// log2 e as they arrive)
+template <typename T, int D, int BT, int NW, bool WRITE_DS>
 __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4 : 2) : 3) mfma_dq_wide(EvoAttnParams p, Extra e) {
+    constexpr bool HAS_BIAS = BT != 0, TILE16 = BT == 2;
     typedef Geo<D> G;
     typedef DqWideGeo<D> R;
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
@@ -79,7 +83,16 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
     const bool bf32 = p.bias_dtype == EVO_F32;
     const char *brow = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h +
                                                (int64_t)qrow * p.bias_stride_row) * (bf32 ? 4 : 2);
+    const unsigned short *btile16 = !TILE16 ? nullptr
+                                    : dead  ? e.bq16 + e.zero_tile + lane * 16
+                                            : e.bq16 + ((((int64_t)bb * p.H + pr.h) * NT + qtc) * NT) * 1024 + lane * 16;
     auto load_btile = [&](int kt, f32x16 &dst) {
+        if constexpr (TILE16) {
+            Tile16 t;
+            load_tile16(btile16 + (dead ? 0 : (int64_t)kt * 1024), t);
+            unpack_tile16<T>(t, dead ? 0.0f : kLog2e, dst);
+            return;
+        }
         if (bdirect) {   // uniform
             const float mul = dead ? 0.0f : kLog2e;
             if (bf32) bias_tile_rows<T, true>(brow, kt * 32, p.N, g, mul, dst);
@@ -269,21 +282,22 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
 // Four waves (128 queries) per workgroup measured faster than eight at every size tried (N = 128
 // .. 2048, all head dims: 114 vs 120 us at N = 256, 298 vs 324 us at N = 1024); bit 0x100 of
 // flags (not part of the public interface) selects eight, for comparison.
-template <typename T, int D, bool HAS_BIAS, bool WRITE_DS>
+template <typename T, int D, int BT, bool WRITE_DS>
 static int dqw_waves(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const int nw = (p.flags & EVO_FLAG_DEBUG_OTHER_WIDTH) ? 8 : 4;
     const unsigned grid = (unsigned)((p.N + nw * 32 - 1) / (nw * 32)) * (unsigned)(p.B * p.H * p.S);
-    if (nw == 8) mfma_dq_wide<T, D, HAS_BIAS, 8, WRITE_DS><<<grid, 512, 0, st>>>(p, e);
-    else mfma_dq_wide<T, D, HAS_BIAS, 4, WRITE_DS><<<grid, 256, 0, st>>>(p, e);
+    if (nw == 8) mfma_dq_wide<T, D, BT, 8, WRITE_DS><<<grid, 512, 0, st>>>(p, e);
+    else mfma_dq_wide<T, D, BT, 4, WRITE_DS><<<grid, 256, 0, st>>>(p, e);
     return hip_rc();
 }
 
 template <typename T, int D>
 static int dqw_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    if (p.bias_dtype == EVO_NONE) return dqw_waves<T, D, false, false>(p, e, st);
-    if (!p.dbias) return dqw_waves<T, D, true, false>(p, e, st);
+    if (p.bias_dtype == EVO_NONE) return dqw_waves<T, D, 0, false>(p, e, st);
+    const bool t16 = e.bq16 && !e.bias_direct;
+    if (!p.dbias) return t16 ? dqw_waves<T, D, 2, false>(p, e, st) : dqw_waves<T, D, 1, false>(p, e, st);
     if (p.S != 1) return EVO_EUNSUPPORTED;   // a sum over S rows is the other kernels' business
-    return dqw_waves<T, D, true, true>(p, e, st);
+    return t16 ? dqw_waves<T, D, 2, true>(p, e, st) : dqw_waves<T, D, 1, true>(p, e, st);
 }
 
 int EVO_CAT(launch_mfma_dqw_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {

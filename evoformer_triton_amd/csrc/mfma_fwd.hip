@@ -18,6 +18,8 @@
 // bias tile (already in log2 units and accumulator order, see prep.hip) is the C operand of
 // the score MFMA, and the mask rides along as three extra columns of K against ones in Q.
 // What is left per score is max, subtract, exp2, add, convert.
+#include <type_traits>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -27,8 +29,13 @@
 
 namespace evo {
 
-template <typename T, int D, bool HAS_BIAS, int NW>
+// BT: 0 no bias; 1 fp32 tiles (times log2 e) or, for very few S rows, the caller's rows; 2 the
+// tiles of a bias in the dtype of q as given (half the bytes per tile, 8 registers in flight
+// instead of 16; unpacked and multiplied by log2 e right before they are used)
+template <typename T, int D, int BT, int NW>
 __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_fwd(EvoAttnParams p, Extra e) {
+    constexpr bool HAS_BIAS = BT != 0, TILE16 = BT == 2;
+    typedef typename std::conditional<TILE16, Tile16, f32x16>::type CTile;   // a bias tile on its way
     constexpr int NTH = NW * 64;                  // threads per workgroup
     constexpr int BQ = NW * 32;                   // query rows per workgroup
     constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round
@@ -106,6 +113,9 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     const char *brow = (const char *)p.bias + ((int64_t)bb * p.bias_stride_b + (int64_t)pr.h * p.bias_stride_h +
                                                (int64_t)qrow * p.bias_stride_row) * (bf32 ? 4 : 2);
     const float bmul = dead ? 0.0f : kLog2e;
+    const unsigned short *btile16 = !TILE16 ? nullptr
+                                    : dead  ? e.bq16 + e.zero_tile + lane * 16
+                                            : e.bq16 + ((((int64_t)bb * p.H + pr.h) * NT + qt) * NT) * 1024 + lane * 16;
 
     float m = -INFINITY, l = 0.0f;
     f32x16 oacc[DT];
@@ -116,8 +126,10 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
 
     // Bias tile kt into 16 registers; past the last tile the previous one is read again
     // (every key there carries the mask floor, so the values do not matter).
-    auto load_btile = [&](int kt, f32x16 &dst) {
-        if (HAS_BIAS && bdirect) {   // uniform
+    auto load_btile = [&](int kt, CTile &dst) {
+        if constexpr (TILE16) {
+            load_tile16(btile16 + (int64_t)min(kt, NT - 1) * bstep, dst);
+        } else if (HAS_BIAS && bdirect) {   // uniform
             if (bf32) bias_tile_rows<T, true>(brow, min(kt, NT - 1) * 32, p.N, g, bmul, dst);
             else bias_tile_rows<T, false>(brow, min(kt, NT - 1) * 32, p.N, g, bmul, dst);
         } else if (HAS_BIAS) {
@@ -163,7 +175,16 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     // One 64-key step: two score tiles, online softmax, four P.V k-steps.  The bias tiles
     // c0, c1 are consumed by the first score MFMAs; the same registers then receive the
     // tiles of the next step, which travel while the softmax and P.V run.
-    auto compute = [&](int step, f32x16 &c0, f32x16 &c1) {
+    auto cval = [&](const CTile &t) -> f32x16 {
+        if constexpr (TILE16) {
+            f32x16 v;
+            unpack_tile16<T>(t, bmul, v);
+            return v;
+        } else {
+            return t;
+        }
+    };
+    auto compute = [&](int step, CTile &c0, CTile &c1) {
         const int kb = (step % SPS) * 64;
         f32x16 a0, a1;
 #pragma unroll
@@ -172,8 +193,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
             v8 k1 = *reinterpret_cast<const v8 *>(&Ks[(kb + 32 + li) * KP + ks * 16 + g * 8]);
             if (ks == 0) {
                 if (HAS_BIAS) {
-                    a0 = Mfma<T>::mma(k0, qf[0], c0);
-                    a1 = Mfma<T>::mma(k1, qf[0], c1);
+                    a0 = Mfma<T>::mma(k0, qf[0], cval(c0));
+                    a1 = Mfma<T>::mma(k1, qf[0], cval(c1));
                 } else {
                     f32x16 z;
 #pragma unroll
@@ -229,7 +250,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     };
 
     const int nsteps = (p.N + 63) / 64;
-    f32x16 c0, c1;
+    CTile c0, c1;
     load_btile(0, c0);
     load_btile(1, c1);
     for (int step = 0; step < nsteps; ++step) {
@@ -277,8 +298,9 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
 template <typename T, int D, int NW>
 static int fwd_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const unsigned nqb = (p.N + NW * 32 - 1) / (NW * 32), grid = nqb * (unsigned)(p.B * p.H * p.S);
-    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, false, NW><<<grid, NW * 64, 0, st>>>(p, e);
-    else mfma_fwd<T, D, true, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    if (p.bias_dtype == EVO_NONE) mfma_fwd<T, D, 0, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    else if (e.bq16 && !e.bias_direct) mfma_fwd<T, D, 2, NW><<<grid, NW * 64, 0, st>>>(p, e);
+    else mfma_fwd<T, D, 1, NW><<<grid, NW * 64, 0, st>>>(p, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }

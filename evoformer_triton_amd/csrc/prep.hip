@@ -6,7 +6,9 @@
 //    (64 lanes x 16 registers contiguous per tile), one with lane = query (for S^T = K Q^T
 //    tiles) and one with lane = key (for S = Q K^T tiles).  A kernel loads a tile straight
 //    into the MFMA accumulator: the bias add of the reference (evoformer.py:68, :450, :594)
-//    becomes the C operand of the score matmul.
+//    becomes the C operand of the score matmul.  A bias in the dtype of q is also stored as
+//    given, 16 bits per entry in the same tile order: the kernels that stream a tile per
+//    score tile read half the bytes and multiply by log2(e) themselves.
 //  * mask -> one row per (b, s), in log2 units, clamped to a finite floor, padded to a
 //    multiple of 32 keys with the floor, each value already split into three 16-bit terms
 //    (hi + mid + lo, exact to 24 bits) of the q/k/v element type.  The kernels carry them as
@@ -37,6 +39,10 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
             const f32x4 z = {0.f, 0.f, 0.f, 0.f};
             *reinterpret_cast<f32x4 *>(e.bq + e.zero_tile + tid * 4) = z;
             *reinterpret_cast<f32x4 *>(e.bk + e.zero_tile + tid * 4) = z;
+            if (e.bq16) {
+                *reinterpret_cast<uint2 *>(e.bq16 + e.zero_tile + tid * 4) = make_uint2(0u, 0u);
+                *reinterpret_cast<uint2 *>(e.bk16 + e.zero_tile + tid * 4) = make_uint2(0u, 0u);
+            }
             return;
         }
         const int kt = t % NT, qt = (t / NT) % NT;
@@ -59,6 +65,20 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
         const int64_t o = ((int64_t)t * 64 + lane) * 16 + 4 * rr;
         *reinterpret_cast<f32x4 *>(e.bq + o) = vq;
         *reinterpret_cast<f32x4 *>(e.bk + o) = vk;
+        if (e.bq16) {
+            // the same entries as given (the bias has the dtype of q: 16 bits, exact)
+            const unsigned short *src = (const unsigned short *)p.bias + base;
+            unsigned wq[4], wk[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int a = 8 * rr + 4 * g + i;
+                const int q1 = qt * 32 + li, key1 = kt * 32 + a, q2 = qt * 32 + a, key2 = kt * 32 + li;
+                wq[i] = (q1 < p.N && key1 < p.N) ? src[(int64_t)q1 * p.bias_stride_row + key1] : 0u;
+                wk[i] = (q2 < p.N && key2 < p.N) ? src[(int64_t)q2 * p.bias_stride_row + key2] : 0u;
+            }
+            *reinterpret_cast<uint2 *>(e.bq16 + o) = make_uint2(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16));
+            *reinterpret_cast<uint2 *>(e.bk16 + o) = make_uint2(wk[0] | (wk[1] << 16), wk[2] | (wk[3] << 16));
+        }
         if (e.bt) {
             // the same four entries of column `key` as given (the dtypes agree, so exact),
             // key-major: N is a multiple of 8 here, so the four are inside the matrix or not
