@@ -80,9 +80,9 @@ static int bias_vec_ok(const EvoAttnParams &p) {
     return aligned(p.bias, a) && p.bias_stride_b % 4 == 0 && p.bias_stride_h % 4 == 0 && p.bias_stride_row % 4 == 0;
 }
 
-// The prepared bias tiles (two fp32 copies in accumulator order) cost 12 bytes of memory traffic
-// per bias entry before any kernel has used one; each kernel then reads 4 bytes per entry and S
-// row.  With very few S rows per (batch, head) - the reference's own speed benchmark has one -
+// The prepared bias tiles (two copies in accumulator order, fp32 or, for a bias in the dtype of q,
+// 16 bits per entry) cost 6 to 12 bytes of memory traffic per bias entry before any kernel has
+// used one; each kernel then reads 2 or 4 bytes per entry and S row.  With very few S rows per (batch, head) - the reference's own speed benchmark has one -
 // the one-workgroup-per-problem kernels read the caller's tensor instead, which needs rows that
 // allow 16-byte (fp32) or 8-byte loads.  EVO_FLAG_DEBUG_BIAS_TILES keeps the tiles, for comparison.
 static bool bias_direct(const EvoAttnParams &p) {
@@ -198,17 +198,19 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
     PrepLayout w{};
     const size_t NT = (size_t)(p.N + 31) / 32;
     w.bias_batches = (p.bias && p.bias_stride_b == 0) ? 1 : p.B;
-    // one extra all-zero tile at the end of each copy
-    const size_t tiles = p.bias && !bias_direct(p) ? ((size_t)w.bias_batches * p.H * NT * NT + 1) * 1024 * 4 : 0;
+    // Bias tiles, with one extra all-zero tile at the end of each copy: for a bias in the dtype of q
+    // the entries as given, 16 bits each (every kernel that reads tiles multiplies by log2 e
+    // itself, in fp32: the product the fp32 tiles hold); else fp32 tiles in log2 units.
+    const bool have_tiles = p.bias && !bias_direct(p);
+    const bool t16_ok = have_tiles && p.bias_dtype == p.dtype && p.dtype != EVO_F32;
+    const size_t tile_elems = have_tiles ? ((size_t)w.bias_batches * p.H * NT * NT + 1) * 1024 : 0;
     size_t off = 0;
-    w.bq = off; off += align_up(tiles);
-    w.bk = off; off += align_up(tiles);
-    // the same tiles in 16 bits for a bias in the dtype of q
-    const bool t16_ok = tiles != 0 && p.bias_dtype == p.dtype && p.dtype != EVO_F32;
+    w.bq = off; off += align_up(t16_ok ? 0 : tile_elems * 4);
+    w.bk = off; off += align_up(t16_ok ? 0 : tile_elems * 4);
     w.bq16 = w.bk16 = (size_t)-1;
     if (t16_ok) {
-        w.bq16 = off; off += align_up(tiles / 2);
-        w.bk16 = off; off += align_up(tiles / 2);
+        w.bq16 = off; off += align_up(tile_elems * 2);
+        w.bk16 = off; off += align_up(tile_elems * 2);
     }
     // transposed 16-bit copy for the kernels that keep bias columns resident
     const bool bt_ok = p.bias && !bias_direct(p) && p.bias_dtype == p.dtype && p.N % 8 == 0;

@@ -82,7 +82,8 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
         for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
 
     const int bb = e.bias_batches > 1 ? b : 0;
-    const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
+    const int64_t tile0 = ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024;
+    const float *btile0 = e.bq + tile0 + lane * 16;
     const float *ztile = e.bq + e.zero_tile + lane * 16;
     // or, for a bias that is used too few times to pay for the tiles, this lane's row of the
     // caller's tensor
@@ -96,6 +97,12 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
             const float mul = dead_row ? 0.0f : kLog2e;
             if (bf32) bias_tile_rows<T, true>(brow, kt * 32, p.N, g, mul, dst);
             else bias_tile_rows<T, false>(brow, kt * 32, p.N, g, mul, dst);
+            return;
+        }
+        if (e.bq16) {   // uniform: a bias in the dtype of q is prepared as given, 16 bits per entry
+            Tile16 t;
+            load_tile16(e.bq16 + (dead_row ? e.zero_tile : tile0 + (int64_t)kt * 1024) + lane * 16, t);
+            unpack_tile16<T>(t, dead_row ? 0.0f : kLog2e, dst);
             return;
         }
         const float *src = dead_row ? ztile : btile0 + (int64_t)kt * 1024;

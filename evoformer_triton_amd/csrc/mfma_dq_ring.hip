@@ -132,14 +132,21 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     f32x16 bres[HAS_BIAS ? NSLOT : 1];
     if (HAS_BIAS) {
         const int bb = e.bias_batches > 1 ? b : 0;
-        const float *btile0 = e.bq + ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
+        // (tiles of a bias in the dtype of q are prepared as given, 16 bits per entry: log2 units here)
+        const int64_t tile0 = ((((int64_t)bb * p.H + h) * NT + qt) * NT) * 1024 + lane * 16;
 #pragma unroll
         for (int j = 0; j < NSLOT; ++j) {
-            const float *src = btile0 + (int64_t)min(slot_tile(j), NT - 1) * 1024;
+            const int64_t o = tile0 + (int64_t)min(slot_tile(j), NT - 1) * 1024;
+            if (e.bq16) {   // uniform
+                Tile16 t;
+                load_tile16(e.bq16 + o, t);
+                unpack_tile16<T>(t, kLog2e, bres[j]);
+            } else {
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
-                const f32x4 v = *reinterpret_cast<const f32x4 *>(src + 4 * rr);
-                bres[j][4 * rr] = v[0]; bres[j][4 * rr + 1] = v[1]; bres[j][4 * rr + 2] = v[2]; bres[j][4 * rr + 3] = v[3];
+                for (int rr = 0; rr < 4; ++rr) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(e.bq + o + 4 * rr);
+                    bres[j][4 * rr] = v[0]; bres[j][4 * rr + 1] = v[1]; bres[j][4 * rr + 2] = v[2]; bres[j][4 * rr + 3] = v[3];
+                }
             }
         }
     }

@@ -2,13 +2,13 @@
 // broadcast operands of the attention, the pair bias and the row mask, into the form the
 // hot loops consume without any per-score arithmetic.
 //
-//  * bias -> two fp32 copies scaled by log2(e) and stored in 32x32 accumulator-tile order
-//    (64 lanes x 16 registers contiguous per tile), one with lane = query (for S^T = K Q^T
-//    tiles) and one with lane = key (for S = Q K^T tiles).  A kernel loads a tile straight
-//    into the MFMA accumulator: the bias add of the reference (evoformer.py:68, :450, :594)
-//    becomes the C operand of the score matmul.  A bias in the dtype of q is also stored as
-//    given, 16 bits per entry in the same tile order: the kernels that stream a tile per
-//    score tile read half the bytes and multiply by log2(e) themselves.
+//  * bias -> two copies in 32x32 accumulator-tile order (64 lanes x 16 registers contiguous
+//    per tile), one with lane = query (for S^T = K Q^T tiles) and one with lane = key (for
+//    S = Q K^T tiles): the bias add of the reference (evoformer.py:68, :450, :594) becomes
+//    the C operand of the score matmul.  An fp32 bias is stored as fp32 scaled by log2(e) and
+//    a kernel loads a tile straight into the MFMA accumulator; a bias in the dtype of q is
+//    stored as given, 16 bits per entry: the kernels read half the bytes and multiply by
+//    log2(e) themselves, in fp32 (the same product).
 //  * mask -> one row per (b, s), in log2 units, clamped to a finite floor, padded to a
 //    multiple of 32 keys with the floor, each value already split into three 16-bit terms
 //    (hi + mid + lo, exact to 24 bits) of the q/k/v element type.  The kernels carry them as
@@ -36,12 +36,13 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
     if (blockIdx.x < n_bias_blocks) {
         const unsigned t = blockIdx.x;
         if (t == n_bias_blocks - 1) {  // the all-zero tile
-            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            *reinterpret_cast<f32x4 *>(e.bq + e.zero_tile + tid * 4) = z;
-            *reinterpret_cast<f32x4 *>(e.bk + e.zero_tile + tid * 4) = z;
             if (e.bq16) {
                 *reinterpret_cast<uint2 *>(e.bq16 + e.zero_tile + tid * 4) = make_uint2(0u, 0u);
                 *reinterpret_cast<uint2 *>(e.bk16 + e.zero_tile + tid * 4) = make_uint2(0u, 0u);
+            } else {
+                const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                *reinterpret_cast<f32x4 *>(e.bq + e.zero_tile + tid * 4) = z;
+                *reinterpret_cast<f32x4 *>(e.bk + e.zero_tile + tid * 4) = z;
             }
             return;
         }
@@ -49,35 +50,36 @@ __global__ void __launch_bounds__(256) prep_kernel(EvoAttnParams p, Extra e, uns
         const int h = (t / NT / NT) % p.H, bb = t / NT / NT / p.H;
         const int li = lane & 31, g = lane >> 5, rr = tid >> 6;
         const int64_t base = (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h;
-        f32x4 vq, vk;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int a = 8 * rr + 4 * g + i;  // accumulator row held by register 4rr+i
-            {
-                const int q = qt * 32 + li, key = kt * 32 + a;
-                vq[i] = (q < p.N && key < p.N) ? kLog2e * bias_at(p, base + (int64_t)q * p.bias_stride_row + key) : 0.0f;
-            }
-            {
-                const int q = qt * 32 + a, key = kt * 32 + li;
-                vk[i] = (q < p.N && key < p.N) ? kLog2e * bias_at(p, base + (int64_t)q * p.bias_stride_row + key) : 0.0f;
-            }
-        }
         const int64_t o = ((int64_t)t * 64 + lane) * 16 + 4 * rr;
-        *reinterpret_cast<f32x4 *>(e.bq + o) = vq;
-        *reinterpret_cast<f32x4 *>(e.bk + o) = vk;
         if (e.bq16) {
-            // the same entries as given (the bias has the dtype of q: 16 bits, exact)
+            // the entries as given (the bias has the dtype of q: 16 bits, exact)
             const unsigned short *src = (const unsigned short *)p.bias + base;
             unsigned wq[4], wk[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int a = 8 * rr + 4 * g + i;
+                const int a = 8 * rr + 4 * g + i;  // accumulator row held by register 4rr+i
                 const int q1 = qt * 32 + li, key1 = kt * 32 + a, q2 = qt * 32 + a, key2 = kt * 32 + li;
                 wq[i] = (q1 < p.N && key1 < p.N) ? src[(int64_t)q1 * p.bias_stride_row + key1] : 0u;
                 wk[i] = (q2 < p.N && key2 < p.N) ? src[(int64_t)q2 * p.bias_stride_row + key2] : 0u;
             }
             *reinterpret_cast<uint2 *>(e.bq16 + o) = make_uint2(wq[0] | (wq[1] << 16), wq[2] | (wq[3] << 16));
             *reinterpret_cast<uint2 *>(e.bk16 + o) = make_uint2(wk[0] | (wk[1] << 16), wk[2] | (wk[3] << 16));
+        } else {
+            f32x4 vq, vk;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int a = 8 * rr + 4 * g + i;
+                {
+                    const int q = qt * 32 + li, key = kt * 32 + a;
+                    vq[i] = (q < p.N && key < p.N) ? kLog2e * bias_at(p, base + (int64_t)q * p.bias_stride_row + key) : 0.0f;
+                }
+                {
+                    const int q = qt * 32 + a, key = kt * 32 + li;
+                    vk[i] = (q < p.N && key < p.N) ? kLog2e * bias_at(p, base + (int64_t)q * p.bias_stride_row + key) : 0.0f;
+                }
+            }
+            *reinterpret_cast<f32x4 *>(e.bq + o) = vq;
+            *reinterpret_cast<f32x4 *>(e.bk + o) = vk;
         }
         if (e.bt) {
             // the same four entries of column `key` as given (the dtypes agree, so exact),

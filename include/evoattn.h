@@ -66,9 +66,9 @@ enum {
     /* Debug switches for A/B comparisons of kernel forms (same results, other kernels); a
      * production caller leaves them clear.  All other bits of `flags` must be zero. */
     EVO_FLAG_DEBUG_OTHER_WIDTH  = 0x100,  /* one-workgroup-per-problem kernels: the other of their two workgroup widths (4 / 8 waves) */
-    EVO_FLAG_DEBUG_NO_KV_RING   = 0x200,
-    EVO_FLAG_DEBUG_FWD_BIAS_TILES = 0x400, /* chunk-of-rows forward: fp32 bias tiles as C operands instead of the caller's 16-bit rows */  /* dK/dV: the one-workgroup-per-problem kernel instead of the chunk-of-rows one */
-    EVO_FLAG_DEBUG_BIAS_TILES   = 0x800,  /* S <= 4: prepare the fp32 bias tiles instead of reading the caller's bias */
+    EVO_FLAG_DEBUG_NO_KV_RING   = 0x200,  /* dK/dV: the one-workgroup-per-problem kernel instead of the chunk-of-rows one */
+    EVO_FLAG_DEBUG_FWD_BIAS_TILES = 0x400, /* chunk-of-rows forward: prepared bias tiles as C operands instead of the caller's 16-bit rows */
+    EVO_FLAG_DEBUG_BIAS_TILES   = 0x800,  /* S <= 4: prepare the bias tiles instead of reading the caller's bias */
     EVO_FLAG_DEBUG_NO_DQ_WIDE   = 0x1000, /* dQ: the kernels that split a row's keys over the waves, also without a dBias sum */
     EVO_FLAG_DEBUG_NO_DQ_SPLIT  = 0x2000  /* dQ + dBias in one kernel, also where dQ and the dBias partials come from two */
 };
@@ -173,7 +173,7 @@ int evoattn_fwd(const EvoAttnParams *p, void *hip_stream);
  * caller's `prep` buffer: `prep` and `prep_bytes` of the parameter block are ignored, o and lse are
  * still the caller's, and the call makes no hipMalloc / hipFree and no allocating library call.
  * Limit: problems whose evoattn_prep_bytes() exceeds EVOATTN_STATIC_PREP_BYTES (16 MiB: rows up to
- * about 512 keys with 8 heads, e.g. B=1 S=512 N=256 H=8 needs 8.3 MB) return EVO_EWORKSPACE.  The
+ * about 512 keys with 8 heads, e.g. B=1 S=512 N=256 H=8 needs 6.0 MB) return EVO_EWORKSPACE.  The
  * array is shared by every call on one GPU (each GPU has its own copy) and keeps the last call's
  * contents: calls that overlap in time on one GPU race on it, so enqueue them on one stream or
  * order them otherwise.  evoattn_bwd cannot reuse this prep (EVO_FLAG_PREP_VALID does not apply). */
