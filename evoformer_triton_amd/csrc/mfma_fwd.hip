@@ -15,12 +15,15 @@
 //
 // The vector ALU, not the matrix core, bounds this kernel (one exp per score), so every
 // addition that can be moved into the matmul is: Q is pre-multiplied by scale*log2(e), the
-// bias tile (already in log2 units and accumulator order, see prep.hip) is the C operand of
-// the score MFMA, and the mask rides along as three extra columns of K against ones in Q.
-// What is left per score is max, subtract, exp2, add, convert.
+// bias tile (in log2 units and accumulator order, see prep.hip) is the C operand of the
+// score MFMA, the mask rides along as three extra columns of K against ones in Q, and the
+// running maximum as three more columns of Q against ones in K, so that after a problem's
+// first 64 keys the scores arrive relative to it.  What is left per score is exp2, an
+// addition and half a conversion; the maximum is searched, and the step rescaled, only in
+// the first step and when a later step's sums show that its maximum moved far.
 #include <type_traits>
 
-#include "common.h"
+#include "bwd_common.h"
 #include "kernels.h"
 
 #ifndef EVO_D
@@ -36,6 +39,11 @@ template <typename T, int D, int BT, int NW>
 __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_fwd(EvoAttnParams p, Extra e) {
     constexpr bool HAS_BIAS = BT != 0, TILE16 = BT == 2;
     typedef typename std::conditional<TILE16, Tile16, f32x16>::type CTile;   // a bias tile on its way
+    // The softmax that skips the search for the maximum after a problem's first 64 keys keeps a
+    // second copy of the score code for the rare step that has to be redone; with fp32 bias
+    // tiles in flight that does not fit 128 registers (8 waves) or 256 at head dim 128, and
+    // those forms keep the plain online softmax.
+    constexpr bool LAZY = BT != 1 || (NW == 4 && D < 128);
     constexpr int NTH = NW * 64;                  // threads per workgroup
     constexpr int BQ = NW * 32;                   // query rows per workgroup
     constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round
@@ -71,7 +79,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
     const int64_t sn = p.stride_n;
     const bool active = q0 < p.N;  // wave-uniform
-    const uint2 *m2row = e.m2 + ((int64_t)pr.b * p.S + pr.s) * npad;
+    const int np256 = (p.N + 255) / 256 * 256;
+    const uint4 *m2arow = e.m2a + ((int64_t)pr.b * p.S + pr.s) * np256;
     const bool dead = e.dead[pr.b * p.S + pr.s] != 0;
 
     // LDS that is read but never staged: the upper half of the mask k-step of K, rows d >= D
@@ -117,7 +126,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
                                     : dead  ? e.bq16 + e.zero_tile + lane * 16
                                             : e.bq16 + ((((int64_t)bb * p.H + pr.h) * NT + qt) * NT) * 1024 + lane * 16;
 
-    float m = -INFINITY, l = 0.0f;
+    float m = LAZY ? 0.0f : -INFINITY, mf = 0.0f, l = 0.0f;
     f32x16 oacc[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -149,12 +158,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
             v8 val = kk < p.N ? ld8(K + (int64_t)kk * sn + ch * 8) : zero8<T>();
             *reinterpret_cast<v8 *>(&Ks[key * KP + ch * 8]) = val;
         }
-        for (int key = tid; key < BKV; key += NTH) {
-            const int kk = kv0 + key;
-            const uint2 mv = kk < npad ? m2row[kk] : pack_split3<T>(kMaskFloor);
-            uint4 aug = {mv.x, mv.y, 0u, 0u};
-            *reinterpret_cast<uint4 *>(&Ks[key * KP + AUGC]) = aug;
-        }
+        for (int key = tid; key < BKV; key += NTH)   // (mask hi, mid, lo, 1, 1, 1, 0, 0); the floor past the padded N
+            *reinterpret_cast<uint4 *>(&Ks[key * KP + AUGC]) = m2arow[min(kv0 + key, np256 - 1)];
         constexpr int NPAIR = BKV / 2;
         for (int it = tid; it < NPAIR * (D / 8); it += NTH) {
             const int ch = it / NPAIR, jp = it % NPAIR, k0 = kv0 + 2 * jp;
@@ -176,7 +181,12 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     // c0, c1 are consumed by the first score MFMAs; the same registers then receive the
     // tiles of the next step, which travel while the softmax and P.V run.
     auto cval = [&](const CTile &t) -> f32x16 {
-        if constexpr (TILE16) {
+        if constexpr (!HAS_BIAS) {
+            f32x16 z;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) z[r] = 0.0f;
+            return z;
+        } else if constexpr (TILE16) {
             f32x16 v;
             unpack_tile16<T>(t, bmul, v);
             return v;
@@ -184,67 +194,141 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
             return t;
         }
     };
-    auto compute = [&](int step, CTile &c0, CTile &c1) {
-        const int kb = (step % SPS) * 64;
-        f32x16 a0, a1;
+    // m is the maximum the probabilities are relative to, mf what the mask k-step subtracts
+    // inside the MFMA (m, or 0 while m is unknown or too large to be carried in three 16-bit
+    // columns next to scores of order one): after a problem's first 64 keys the scores leave
+    // the matrix core relative to m and the common step neither searches its maximum nor
+    // subtracts.
+    // one 32-key score tile (keys kb .. kb + 31 of the stage) on top of its bias tile
+    auto score1 = [&](int kb, const f32x16 &bias, f32x16 &a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            v8 k0 = *reinterpret_cast<const v8 *>(&Ks[(kb + li) * KP + ks * 16 + g * 8]);
-            v8 k1 = *reinterpret_cast<const v8 *>(&Ks[(kb + 32 + li) * KP + ks * 16 + g * 8]);
-            if (ks == 0) {
-                if (HAS_BIAS) {
-                    a0 = Mfma<T>::mma(k0, qf[0], cval(c0));
-                    a1 = Mfma<T>::mma(k1, qf[0], cval(c1));
-                } else {
-                    f32x16 z;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) z[r] = 0.0f;
-                    a0 = Mfma<T>::mma(k0, qf[0], z);
-                    a1 = Mfma<T>::mma(k1, qf[0], z);
-                }
-            } else {
-                a0 = Mfma<T>::mma(k0, qf[ks], a0);
-                a1 = Mfma<T>::mma(k1, qf[ks], a1);
-            }
-            if (RESID && ks < KSD) {
-                a0 = Mfma<T>::mma(k0, qlo[ks], a0);
-                a1 = Mfma<T>::mma(k1, qlo[ks], a1);
-            }
+            v8 k = *reinterpret_cast<const v8 *>(&Ks[(kb + li) * KP + ks * 16 + g * 8]);
+            a = Mfma<T>::mma(k, qf[ks], ks == 0 ? bias : a);
+            if (RESID && ks < KSD) a = Mfma<T>::mma(k, qlo[ks], a);
         }
-        load_btile(2 * step + 2, c0);
-        load_btile(2 * step + 3, c1);
+    };
+    // where the maximum stands; `used` is the mf the step's scores were formed with
+    auto settle = [&](bool first, f32x16 &a0, f32x16 &a1, float used) {
         float mloc = fmaxf(a0[0], a1[0]);
 #pragma unroll
         for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        const bool grow = mloc > m + TAU;
-        if (__any(grow)) {
-            const float mn = grow ? mloc : m;
-            const float alpha = fast_exp2(m - mn);
-            l *= alpha;
-            m = mn;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+        {   // exchange between the two lane groups without touching LDS
+            const unsigned u = __float_as_uint(mloc);
+            auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            mloc = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
         }
-        float psum = 0.0f;
+        const float cand = mloc + used;
+        // move m only when the maximum grows by more than 2^TAU (always at the first step)
+        const bool grow = first || cand > m + TAU;
+        if (__any(grow || m != used)) {
+            const float mn = grow ? cand : m;
+            if (!first) {
+                const float alpha = fast_exp2(m - mn);   // <= 1; 1 where this lane's m stays
+                l *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+            }
+            m = mn;
+            const float dsub = m - used;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                a0[r] -= dsub;
+                a1[r] -= dsub;
+            }
+            // from the next scores on the MFMA subtracts m itself
+            mf = fabsf(m) <= 1024.0f ? m : 0.0f;
+            const v8 qa = aug8<T>(ones3<T>(), pack_split3<T>(-mf));   // ones x mask columns, -mf x ones
+            if (g == (AUG_IN_PAD ? 1 : 0)) qf[KS - 1] = qa;
+        }
+    };
+    // P = exp2 and this lane's sum of them in fp32 (the reference sums before it rounds,
+    // evoformer.py:77-84: the log-sum-exp the backward normalises with carries no rounding of
+    // P, which on a peaked row would be a relative 2^-9 on every gradient), then P rounded to T
+    auto probs = [&](f32x16 &a0, f32x16 &a1, v8 (&pf)[4], float &ls) {
+        ls = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            a0[r] = fast_exp2(a0[r] - m);
-            a1[r] = fast_exp2(a1[r] - m);
-            psum += a0[r] + a1[r];
+            a0[r] = fast_exp2(a0[r]);
+            a1[r] = fast_exp2(a1[r]);
+            ls += a0[r] + a1[r];
         }
-        l += psum;
+#pragma unroll
+        for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[ts][i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+    };
+    auto compute = [&](int step, CTile &c0, CTile &c1) {
+        const int kb = (step % SPS) * 64;
+        const float used = mf;
+        f32x16 a0, a1;
+        score1(kb, cval(c0), a0);
+        score1(kb + 32, cval(c1), a1);
+        load_btile(2 * step + 2, c0);
+        load_btile(2 * step + 3, c1);
+        if constexpr (!LAZY) {
+            // the plain online softmax: maximum of every step, subtraction, fp32 row sums
+            float mloc = fmaxf(a0[0], a1[0]);
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, fmaxf(a0[r], a1[r]));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+            const bool grow = mloc > m + TAU;
+            if (__any(grow)) {
+                const float mn = grow ? mloc : m;
+                const float alpha = fast_exp2(m - mn);
+                l *= alpha;
+                m = mn;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+            }
+            float psum = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                a0[r] = fast_exp2(a0[r] - m);
+                a1[r] = fast_exp2(a1[r] - m);
+                psum += a0[r] + a1[r];
+            }
+            l += psum;
+#pragma unroll
+            for (int ts = 0; ts < 4; ++ts) {
+                v8 pf1;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pf1[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    v8 va = *reinterpret_cast<const v8 *>(&Vt[(dt * 32 + li) * VP + kb + ts * 16 + g * 8]);
+                    oacc[dt] = Mfma<T>::mma(va, pf1, oacc[dt]);
+                }
+            }
+            return;
+        }
+        v8 pf[4];
+        float ls;
+        const bool lazy = step != 0 && !__any(m != used);
+        if (!lazy) settle(step == 0, a0, a1, used);
+        probs(a0, a1, pf, ls);
+        // A lane sum beyond 2^13 (or not a number) means some score stands far above m: the step
+        // is then redone the long way, from the bias tiles read again.
+        if (__builtin_expect(lazy && __any(!(ls <= 8192.0f)), 0)) {
+            CTile t;
+            load_btile(2 * step, t);
+            score1(kb, cval(t), a0);
+            load_btile(2 * step + 1, t);
+            score1(kb + 32, cval(t), a1);
+            settle(false, a0, a1, used);
+            probs(a0, a1, pf, ls);
+        }
+        l += ls;
 #pragma unroll
         for (int ts = 0; ts < 4; ++ts) {
-            v8 pf;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) pf[i] = (T)((ts < 2 ? a0 : a1)[8 * (ts & 1) + i]);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 v8 va = *reinterpret_cast<const v8 *>(&Vt[(dt * 32 + li) * VP + kb + ts * 16 + g * 8]);
-                oacc[dt] = Mfma<T>::mma(va, pf, oacc[dt]);
+                oacc[dt] = Mfma<T>::mma(va, pf[ts], oacc[dt]);
             }
         }
     };
