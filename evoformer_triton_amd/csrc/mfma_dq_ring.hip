@@ -34,8 +34,9 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // QT: 32-row query tiles per workgroup (2, or 1 for rows of several key blocks: half the
 // resident bias tiles and dBias accumulators per wave).
-// KB: keys per stage (256, or 128: for head dim 64, whose rows are long, and for rows of 257..384
-// keys, which three blocks of 128 cover without an empty half block).
+// KB: keys per stage (256; 128 for head dim 64, whose rows are long, and at head dim 32 for rows of
+// 257..384 keys, which three blocks of 128 cover without an empty half block; 384 for such rows at
+// head dims 8 and 16, where a whole row fits one stage).
 template <int D, int QT, int KB>
 struct RingGeo {
     static constexpr int C = D / 8;                          // 16-byte chunks per row
@@ -518,8 +519,12 @@ static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 // and 16 of dBias sums (three tiles per wave fit, four spill and run slower than the
 // one-workgroup-per-problem kernel):
 //   head dims 8, 16, 32   N <= 256        1 block of 256 keys, 2 query tiles per workgroup (2 tiles per wave)
+//   head dims 8, 16       N <= 384        1 block of 384 keys, 2 query tiles               (3 tiles per wave; one stage and two
+//                                         barriers per row: at head dim 16, S = 512, H = 8, N = 384 260 us against 330 us
+//                                         for three blocks of 128 keys, at head dim 8, S = 1024 457 against 467 us for two
+//                                         blocks of 256; at head dim 32 its stage and tiles together spill 113 registers)
 //   head dim 8            N <= 512        2 blocks of 256 keys, 2 query tiles               (4 tiles per wave; its working set is small)
-//   head dims 16, 32      N <= 384        3 blocks of 128 keys, 2 query tiles               (3 tiles per wave; measured
+//   head dim 32           N <= 384        3 blocks of 128 keys, 2 query tiles               (3 tiles per wave; measured
 //                                         196 us against 256 us for the next form at N = 384, D = 32, S = 384, H = 4)
 //                         N <= 512, 768   2, 3 blocks of 256 keys, 1 query tile             (2, 3 tiles per wave)
 //   head dim 64           N <= 128        1 block of 128 keys, 2 query tiles                (1 tile per wave)
@@ -530,8 +535,8 @@ template <int D>
 constexpr DqrForm dqr_form(int n) {
     if (D == 64) return n <= 128 ? DqrForm{1, 2, 128} : DqrForm{0, 0, 0};
     if (n <= 256) return DqrForm{1, 2, 256};
-    if (D == 8) return n <= 512 ? DqrForm{2, 2, 256} : DqrForm{0, 0, 0};
-    if (n <= 384) return DqrForm{3, 2, 128};
+    if (D == 8) return n <= 384 ? DqrForm{1, 2, 384} : n <= 512 ? DqrForm{2, 2, 256} : DqrForm{0, 0, 0};
+    if (n <= 384) return D == 16 ? DqrForm{1, 2, 384} : DqrForm{3, 2, 128};
     if (n <= 512) return DqrForm{2, 1, 256};
     if (n <= 768) return DqrForm{3, 1, 256};
     return DqrForm{0, 0, 0};
@@ -543,11 +548,16 @@ static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     if constexpr (D == 64) {
         if (f.nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2, 128>(p, e, st);
     } else {
-        if (f.nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2, 256>(p, e, st);
+        if (f.nblk == 1 && f.kb == 256) return dqr_launch<T, D, HAS_BIAS, 1, 2, 256>(p, e, st);
         if constexpr (D == 8) {
+            if (f.nblk == 1 && f.kb == 384) return dqr_launch<T, D, HAS_BIAS, 1, 2, 384>(p, e, st);
             if (f.nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 2, 256>(p, e, st);
         } else {
-            if (f.nblk == 3 && f.kb == 128) return dqr_launch<T, D, HAS_BIAS, 3, 2, 128>(p, e, st);
+            if constexpr (D == 16) {
+                if (f.nblk == 1 && f.kb == 384) return dqr_launch<T, D, HAS_BIAS, 1, 2, 384>(p, e, st);
+            } else {
+                if (f.nblk == 3 && f.kb == 128) return dqr_launch<T, D, HAS_BIAS, 3, 2, 128>(p, e, st);
+            }
             if (f.nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 1, 256>(p, e, st);
             if (f.nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3, 1, 256>(p, e, st);
         }

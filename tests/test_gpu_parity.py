@@ -332,7 +332,9 @@ def test_small_cases_fp16(E, case):
 
 @pytest.mark.parametrize("shape,mask", [((1, 37, 256, 2, 32), "add"), ((1, 5, 200, 3, 16), "bool"),
                                         ((2, 3, 130, 2, 8), "soft"), ((1, 4, 384, 2, 32), "add"),
-                                        ((1, 3, 480, 1, 64), "add")])
+                                        ((1, 3, 480, 1, 64), "add"),
+                                        # rows of 257..384 keys at head dims 8 and 16: one 384-key stage in the dQ kernel
+                                        ((1, 6, 384, 2, 16), "add"), ((1, 5, 328, 2, 16), "bool"), ((1, 6, 376, 3, 8), "soft")])
 def test_chunk_of_rows_kernels_match_per_problem_kernels(E, shape, mask):
     """The forms that walk over a chunk of S rows and the one-workgroup-per-problem forms do
     the same arithmetic up to the order of a few fp32 additions: results agree to a
