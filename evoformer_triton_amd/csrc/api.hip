@@ -129,6 +129,11 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     const int min_s = p.N > 2048 ? 2 : p.D == 32 && p.N > 512 ? 8 : 64;   // (beyond 2048 keys the one kernel has no form at all)
     const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
     if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
+    // Rows that fill the one kernel's key blocks exactly stay with it (bf16, H = 4, S = N, backward: N = 384 293
+    // against 299 us, N = 512 588 against 648 us, N = 768 2.00 against 2.05 ms; head dim 16, N = 768: 1.09 against
+    // 1.15 ms); with a partly empty last block the pair wins (N = 320: 108 against 121 us, N = 640: 1.02 against 1.07 ms).
+    const bool whole_blocks = p.N % 256 == 0 || (p.N <= 384 && p.N % 128 == 0);
+    if (whole_blocks && dq_ring_ok(p)) return false;
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }
