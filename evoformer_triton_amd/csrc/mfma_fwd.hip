@@ -41,9 +41,12 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     typedef typename std::conditional<TILE16, Tile16, f32x16>::type CTile;   // a bias tile on its way
     // The softmax that skips the search for the maximum after a problem's first 64 keys keeps a
     // second copy of the score code for the rare step that has to be redone; with fp32 bias
-    // tiles in flight that does not fit 128 registers (8 waves) or 256 at head dim 128, and
-    // those forms keep the plain online softmax.
-    constexpr bool LAZY = BT != 1 || (NW == 4 && D < 128);
+    // tiles in flight that does not fit 128 registers (8 waves) or 256 at head dim 128, and in
+    // the 4-wave forms it measured no better on balance (B = 4, S = 1, H = 32, D = 64, fp32 bias
+    // read from the caller's rows: N = 1024 136 against 130 TFLOP/s, N = 768 107 against 130):
+    // the forms with an fp32 bias keep the plain online softmax, and so do head dims 64 and 128
+    // (no bias, B = 4, S = 1, H = 32, D = 64, N = 1024: 72 against 62 us).
+    constexpr bool LAZY = BT != 1 && D <= 32;
     constexpr int NTH = NW * 64;                  // threads per workgroup
     constexpr int BQ = NW * 32;                   // query rows per workgroup
     constexpr int BKV = D <= 32 ? 256 : 128;      // keys staged per round
