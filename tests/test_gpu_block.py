@@ -1,0 +1,99 @@
+"""The attention block around the kernels (projections in, fused gate, projection out) against
+the same block in plain torch: outputs and every gradient, in bf16 against an fp32 copy of
+the module, next to what plain torch in bf16 makes of the same block."""
+import copy
+import os
+import sys
+
+import pytest
+import torch
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+pytestmark = pytest.mark.gpu
+
+
+def _grads(block, out, m, z, dout):
+    block.zero_grad(set_to_none=True)
+    m.grad = None
+    if z is not None:
+        z.grad = None
+    out.backward(dout)
+    g = {"m": m.grad.float().clone()}
+    if z is not None:
+        g["z"] = z.grad.float().clone()
+    for n, p in block.named_parameters():
+        g[n] = p.grad.float().clone()
+    return g
+
+
+@pytest.mark.parametrize("case", [(1, 12, 256, 4, 32, 64, 32, True, True),     # chunk-of-rows kernels
+                                  (2, 5, 100, 2, 16, 32, 16, True, True),      # ragged rows, two batches
+                                  (1, 6, 384, 4, 32, 64, None, False, True),   # no pair bias
+                                  (1, 4, 128, 8, 8, 64, 16, True, False)],     # no gate, head dim 8
+                         ids=lambda c: "-".join(map(str, c)))
+def test_block_matches_plain_torch(case):
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    B, S, N, H, D, c_m, c_z, with_mask, gating = case
+    dev = torch.device("cuda", torch.cuda.current_device())
+    torch.manual_seed(11)
+    ref = GatedAttentionBlock(c_m, D, H, c_z=c_z, gating=gating).to(dev)
+    with torch.no_grad():                     # default initialisation gives near-uniform attention: sharpen it
+        for lin in (ref.linear_q, ref.linear_k):
+            lin.weight.mul_(3.0)
+    blk = copy.deepcopy(ref).to(torch.bfloat16)
+    ref = copy.deepcopy(blk).float()          # the same (bf16-representable) parameters in fp32
+    m32 = torch.randn(B, S, N, c_m, device=dev)
+    z32 = torch.randn(B, N, N, c_z, device=dev) if c_z else None
+    mask = (torch.rand(B, S, N, device=dev) < 0.9).float() if with_mask else None
+    dout32 = torch.randn(B, S, N, c_m, device=dev)
+    m16 = m32.to(torch.bfloat16).requires_grad_()
+    z16 = z32.to(torch.bfloat16).requires_grad_() if c_z else None
+    m32 = m16.detach().float().requires_grad_()
+    z32 = z16.detach().float().requires_grad_() if c_z else None
+    dout16 = dout32.to(torch.bfloat16)
+
+    o_ref = ref.forward_eager(m32, z32, mask)
+    g_ref = _grads(ref, o_ref, m32, z32, dout16.float())
+    o_hip = blk(m16, z16, mask)
+    g_hip = _grads(blk, o_hip, m16, z16, dout16)
+    o_eag = blk.forward_eager(m16, z16, mask)
+    g_eag = _grads(blk, o_eag, m16, z16, dout16)
+
+    def err(a, b):
+        return (a.float() - b.float()).abs().max().item()
+
+    # The block is a chain of bf16 operations (LayerNorm, five GEMMs); its distance to fp32 is
+    # set by those, not by the attention kernels: the path through the kernels has to be as
+    # close to the fp32 block as plain torch in bf16 is (within a factor and a floor), on the
+    # output and on every gradient.
+    scale = max(1.0, o_ref.abs().max().item())
+    assert err(o_hip, o_ref) <= max(2.0 * err(o_eag, o_ref), 2e-2 * scale), ("out", err(o_hip, o_ref), err(o_eag, o_ref))
+    def rel(a, b):
+        return ((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-12)).item()
+
+    for n in g_ref:
+        assert torch.isfinite(g_hip[n]).all(), n
+        # every gradient is a sum over many 16-bit roundings (of dBias entries, of GEMM outputs):
+        # the measure is its distance to the fp32 gradient relative to that gradient's norm
+        r_hip, r_eag = rel(g_hip[n], g_ref[n]), rel(g_eag[n], g_ref[n])
+        e_hip, e_eag = err(g_hip[n], g_ref[n]), err(g_eag[n], g_ref[n])
+        print(f"{n}: rel L2 error {r_hip:.2e} (plain torch in bf16: {r_eag:.2e}), max-abs {e_hip:.2e} ({e_eag:.2e})")
+        # (the bias of the pair LayerNorm shifts every score of a head alike: its exact gradient
+        # is zero and what either path returns is rounding noise, judged by its size alone)
+        assert r_hip <= max(2.0 * r_eag, 2e-2) or e_hip <= max(4.0 * e_eag, 2e-2), (n, r_hip, r_eag, e_hip, e_eag)
+
+
+def test_block_operands_are_views_of_the_projections():
+    """Q, K, V and the gate reach the kernels without a copy: contiguous [B,S,N,H,D] views of
+    the projections' [B,S,N,H*D] results."""
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    dev = torch.device("cuda", torch.cuda.current_device())
+    blk = GatedAttentionBlock(32, 16, 2, c_z=8).to(dev).to(torch.bfloat16)
+    m = torch.randn(1, 3, 40, 32, device=dev, dtype=torch.bfloat16)
+    z = torch.randn(1, 40, 40, 8, device=dev, dtype=torch.bfloat16)
+    q, k, v, g, add_mask, bias = blk.operands(m, z, torch.ones(1, 3, 40, device=dev))
+    for t in (q, k, v, g):
+        assert t.is_contiguous() and tuple(t.shape) == (1, 3, 40, 2, 16)
+    assert tuple(bias.shape) == (1, 1, 2, 40, 40) and bias.dtype == torch.bfloat16 and bias.is_contiguous()
+    assert tuple(add_mask.shape) == (1, 3, 1, 1, 40) and float(add_mask.abs().max()) == 0.0
