@@ -77,7 +77,8 @@ __device__ __forceinline__ float pair_sums(typename Mfma<T>::v8 x, float acc) {
 }
 
 // BIASK: 0 no bias, 1 fp32 tiles (x log2(e), accumulator order) as C operands, 2 the caller's 16-bit rows through the identity
-template <typename T, int D, int BIASK>
+// GATED: the output gate in the epilogue (a kernel of its own: the ungated one carries none of its registers)
+template <typename T, int D, int BIASK, bool GATED>
 __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     typedef FwdRingGeo<D> R;
     constexpr int C = R::C;
@@ -472,12 +473,14 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 if (g == 0) p.lse[(int64_t)pid * p.N + q] = (m + __log2f(l)) * kLn2;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) store_row_tile<T>(O, dt * 32, D, oacc[dt], inv, g);
-                if (p.gate) {   // uniform: sigmoid(gate) * O goes out as a second tensor, from the same registers
+                if constexpr (GATED) {   // sigmoid(gate) * O goes out as a second tensor, from the same registers
                     const int64_t off = base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) oacc[dt][r] *= inv;
+                        // (asked for here and not ahead of the row's stores: eight more registers across the
+                        // stash cost the kernel 7 more spilled registers and 14 us, 150 against 136 us)
                         gate_row_tile<T>((const T *)p.gate + off, dt * 32, D, oacc[dt], g);
                         store_row_tile<T>((T *)p.o_gated + off, dt * 32, D, oacc[dt], 1.0f, g);
                     }
@@ -491,12 +494,12 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, int BIASK>
-static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
+template <typename T, int D, int BIASK, bool GATED>
+static int fwdr_launch_g(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
     typedef FwdRingGeo<D> R;
     static PerDevice done{};
     int cus = 256;
-    auto kern = mfma_fwd_ring<T, D, BIASK>;
+    auto kern = mfma_fwd_ring<T, D, BIASK, GATED>;
     if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, &cus)) return rc;
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     Extra e = e0;
@@ -509,6 +512,11 @@ static int fwdr_launch(const EvoAttnParams &p, const Extra &e0, hipStream_t st) 
     kern<<<(unsigned)bh * (unsigned)e.n_chunks, 512, R::LDS_BYTES, st>>>(p, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
+}
+
+template <typename T, int D, int BIASK>
+static int fwdr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
+    return p.gate ? fwdr_launch_g<T, D, BIASK, true>(p, e, st) : fwdr_launch_g<T, D, BIASK, false>(p, e, st);
 }
 
 template <typename T>
