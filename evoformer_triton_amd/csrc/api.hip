@@ -150,9 +150,9 @@ static bool dq_writes_dbias(const EvoAttnParams &p) { return p.dbias && p.S == 1
 
 // S is split into chunks; one workgroup of the dQ kernel sums dS over one chunk and
 // writes one partial dBias tile.  Enough chunks to fill the chip, no more.  The kernel that
-// walks over its chunk with one workgroup per CU (256 CUs) wants the workgroups to come in
-// whole rounds: among the chunk counts that give one to four rounds it takes the one that
-// leaves the fewest CUs idle in the last round (ties: the fewest chunks).
+// walks over its chunk with one workgroup per CU (256 CUs) runs in rounds of 256 workgroups:
+// among the chunk counts that give up to four rounds it takes the cheapest by a count of rows
+// per workgroup, rounds and partials (below).
 static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t NT = (p.N + 31) / 32;
     if (dq_split_ok(p)) {
@@ -179,13 +179,19 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     const int64_t base = (ring ? (p.N + mfma_dqr_qrows(p.D, p.N) - 1) / mfma_dqr_qrows(p.D, p.N) : NT) * p.B * p.H;
     int64_t want = (1024 + base - 1) / base;
     if (ring) {
+        // One workgroup per CU at a time: n chunks take ceil(base n / 256) rounds of ceil(S / n) rows each.
+        // A round also costs its start, its resident bias, its partials and the spread of its
+        // workgroups' finishing times, about three rows' worth (8-9 us measured), and every chunk a
+        // partial dBias to write and to sum again, about a quarter of a row: S = N = 384, H = 4 takes 10
+        // chunks in one round (240 workgroups) over 32 in three full rounds (backward 269 against 298 us),
+        // S = N = 768 8 chunks in three rounds over 5 in two (2.00 against 2.01 ms).
         constexpr int64_t CUS = 256;
-        const int64_t lo = (CUS + base - 1) / base, hi = (4 * CUS + base - 1) / base;
-        double best = -1.0;
-        for (int64_t n = lo; n <= hi; ++n) {
-            const int64_t wgs = base * n, rounds = (wgs + CUS - 1) / CUS;
-            const double eff = (double)wgs / (double)(rounds * CUS);
-            if (eff > best + 1e-9) { best = eff; want = n; }
+        const int64_t hi = (4 * CUS + base - 1) / base;
+        double best = 1e30;
+        for (int64_t n = 1; n <= hi && n <= p.S; ++n) {
+            const int64_t rounds = (base * n + CUS - 1) / CUS, rows = (p.S + n - 1) / n;
+            const double cost = (double)rounds * (double)rows + 3.0 * (double)rounds + 0.25 * (double)n;
+            if (cost < best - 1e-9) { best = cost; want = n; }
         }
     }
     if (want < 1) want = 1;
