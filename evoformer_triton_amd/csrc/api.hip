@@ -178,22 +178,11 @@ static void chunking(const EvoAttnParams &p, int *n_chunks, int *chunk) {
     // workgroups per chunk: one per slab of query rows and head
     const int64_t base = (ring ? (p.N + mfma_dqr_qrows(p.D, p.N) - 1) / mfma_dqr_qrows(p.D, p.N) : NT) * p.B * p.H;
     int64_t want = (1024 + base - 1) / base;
-    if (ring) {
-        // One workgroup per CU at a time: n chunks take ceil(base n / 256) rounds of ceil(S / n) rows each.
-        // A round also costs its start, its resident bias, its partials and the spread of its
-        // workgroups' finishing times, about three rows' worth (8-9 us measured), and every chunk a
-        // partial dBias to write and to sum again, about a quarter of a row: S = N = 384, H = 4 takes 10
-        // chunks in one round (240 workgroups) over 32 in three full rounds (backward 269 against 298 us),
-        // S = N = 768 8 chunks in three rounds over 5 in two (2.00 against 2.01 ms).
-        constexpr int64_t CUS = 256;
-        const int64_t hi = (4 * CUS + base - 1) / base;
-        double best = 1e30;
-        for (int64_t n = 1; n <= hi && n <= p.S; ++n) {
-            const int64_t rounds = (base * n + CUS - 1) / CUS, rows = (p.S + n - 1) / n;
-            const double cost = (double)rounds * (double)rows + 3.0 * (double)rounds + 0.25 * (double)n;
-            if (cost < best - 1e-9) { best = cost; want = n; }
-        }
-    }
+    // The kernel over a chunk of rows: every chunk is a partial dBias to write and to sum again, about a
+    // quarter of a row's worth (S = N = 384, H = 4 takes 10 chunks in one round of 240 workgroups over 32 in
+    // three full rounds: backward 269 against 298 us; S = N = 768 8 chunks in three rounds over 5 in two:
+    // 2.00 against 2.01 ms).
+    if (ring) want = chunks_for_rounds(base, p.S, 256, 0.25);
     if (want < 1) want = 1;
     if (want > p.S) want = p.S;
     *chunk = (int)((p.S + want - 1) / want);

@@ -57,6 +57,25 @@ struct Extra {
     long long *trace;  // trace builds only: 16 timestamps per wave
 };
 
+// Rows of S per workgroup for a kernel that walks over a chunk of S rows of one of `base`
+// (batch, head, query slab) items with one workgroup per CU at a time: n chunks run in
+// ceil(base n / cus) rounds of ceil(S / n) rows.  A round also costs its start, its resident
+// bias and the spread of its workgroups' finishing times, about three rows' worth, and a
+// chunk `per_chunk` rows' worth (a partial result to write and sum again, where there is one).
+// Returns the number of chunks with the smallest such count, among those of up to four rounds.
+static inline int chunks_for_rounds(int64_t base, int S, int cus, double per_chunk) {
+    if (base < 1) base = 1;
+    const int64_t hi = (4 * (int64_t)cus + base - 1) / base;
+    int64_t want = 1;
+    double best = 1e30;
+    for (int64_t n = 1; n <= hi && n <= S; ++n) {
+        const int64_t rounds = (base * n + cus - 1) / cus, rows = (S + n - 1) / n;
+        const double cost = (double)rounds * (double)rows + 3.0 * (double)rounds + per_chunk * (double)n;
+        if (cost < best - 1e-9) { best = cost; want = n; }
+    }
+    return (int)want;
+}
+
 // Linear block id -> logical id such that consecutive logical ids run on one XCD
 // (hardware deals consecutive workgroup ids round-robin over the 8 XCDs, each with its
 // own L2).  Bijection on [0,total) for any total.

@@ -504,9 +504,7 @@ static int fwdr_launch_g(const EvoAttnParams &p, const Extra &e0, hipStream_t st
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     Extra e = e0;
     const int bh = p.B * p.H;
-    int want = (cus + bh - 1) / bh;
-    if (want < 1) want = 1;
-    if (want > p.S) want = p.S;
+    const int want = chunks_for_rounds(bh, p.S, cus, 0.0);
     e.chunk = (p.S + want - 1) / want;
     e.n_chunks = (p.S + e.chunk - 1) / e.chunk;
     kern<<<(unsigned)bh * (unsigned)e.n_chunks, 512, R::LDS_BYTES, st>>>(p, e);
