@@ -111,29 +111,25 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
     return !(p.flags & (EVO_FLAG_PER_PROBLEM | EVO_FLAG_DEBUG_NO_DQ_WIDE)) && (int64_t)((p.N + 127) / 128) * p.B * p.H * p.S >= 32;
 }
 
-// Rows of more than 384 keys with a dBias to sum (up to there the dQ kernel that keeps the sums
-// has two query tiles per workgroup, beyond one; with at most four (batch, head) pairs, where
-// that kernel fills the chip only with many chunks of S and so many partials, from 257 keys
-// on: S = N = 384, H = 4: backward 322 against 364 us, with H = 8 857 against 827 us): dQ from that same kernel, and the dBias
-// partials from a kernel of their own that forms dS a second time (dQ and partials, S = N:
-// N = 512: 436 against 483 us, N = 768: 1.32 against 1.67 ms, N = 1024, S = 256: 0.80 against
-// 1.56 ms; N = 384: 211 against 204 us, and with few S rows the second kernel's start-up shows;
-// head dims 8 and 16, whose one-kernel form reaches to N = 512: 569 against 367 us and 696
-// against 661 us there, 0.65 against 1.38 ms and 740 against 793 us at N = 768).
+// Long rows with a dBias to sum: either the dQ kernel over a chunk of rows, which keeps the sums of its key
+// tiles next to dQ (up to 512 keys with two query tiles per workgroup or in one or two stages, beyond in
+// blocks of 256 keys with one query tile), or dQ from the kernel whose waves own their query rows for all keys
+// and the dBias partials from a kernel of their own that forms dS a second time.  The pair is taken where
+// the one kernel has no form (beyond 768 keys; head dim 64 beyond 128 keys; head dim 8 beyond 512) and, between
+// 513 and 768 keys, where the row leaves the one kernel's last 256-key block mostly empty.  Whole backward,
+// bf16, H = 4, head dim 32, one kernel / the pair: N = 320 (S = 128) 92 / 110 us; N = 352, 448, 480 (S = 256)
+// 177 / 190, 259 / 274, 277 / 291 us; N = 576, 704, 736 (S = 256) 459 / 436, 633 / 623, 660 / 654 us; N = 640
+// (B = 2, S = 256) 1.06 / 0.99 ms; head dim 16, H = 8, S = 512: N = 576 1.51 / 1.46 ms, N = 640 1.72 / 1.63 ms,
+// N = 704 2.01 / 2.06 ms.
 // EVO_FLAG_DEBUG_NO_DQ_SPLIT selects the one kernel, for comparison.
 static bool dq_split_ok(const EvoAttnParams &p) {
-    // shortest rows that go this way: where the kernel that keeps the sums has no form with
-    // prefetch (head dim 64 beyond 128 keys) or measured slower
-    // fewest S rows: the second kernel's start-up has to pay (N = 768, D = 32: ahead from 8 rows on;
-    // N = 512: 72 against 66 us at 32 rows)
+    // fewest S rows: the second kernel's start-up has to pay (N = 768, D = 32: ahead from 8 rows on)
     const int min_s = p.N > 2048 ? 2 : p.D == 32 && p.N > 512 ? 8 : 64;   // (beyond 2048 keys the one kernel has no form at all)
-    const int min_n = p.D == 64 ? 128 : p.D != 32 ? 512 : p.B * p.H <= 4 ? 256 : 384;
+    const int min_n = p.D == 64 ? 128 : 512;
     if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
-    // Rows that fill the one kernel's key blocks exactly stay with it (bf16, H = 4, S = N, backward: N = 384 293
-    // against 299 us, N = 512 588 against 648 us, N = 768 2.00 against 2.05 ms; head dim 16, N = 768: 1.09 against
-    // 1.15 ms); with a partly empty last block the pair wins (N = 320: 108 against 121 us, N = 640: 1.02 against 1.07 ms).
-    const bool whole_blocks = p.N % 256 == 0 || (p.N <= 384 && p.N % 128 == 0);
-    if (whole_blocks && dq_ring_ok(p)) return false;
+    const int rem = p.N % 256;
+    const bool full_blocks = rem == 0 || rem >= (p.D == 32 ? 224 : 192);
+    if (full_blocks && dq_ring_ok(p)) return false;
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }

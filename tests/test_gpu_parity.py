@@ -416,15 +416,15 @@ def test_dq_where_no_dbias_is_asked_for(E, case):
         assert max_err(got[name], other[name]) <= ulp * max(1.0, other[name].abs().max().item()), name
 
 
-@pytest.mark.parametrize("case", [(1, 64, 416, 1, 32, "add", torch.bfloat16), (1, 70, 520, 2, 16, "bool", torch.bfloat16),
-                                  (1, 64, 530, 1, 8, "soft", torch.float16), (2, 66, 400, 1, 32, "bool", torch.float16),
+@pytest.mark.parametrize("case", [(1, 64, 544, 1, 32, "add", torch.bfloat16), (1, 70, 520, 2, 16, "bool", torch.bfloat16),
+                                  (1, 64, 530, 1, 8, "soft", torch.float16), (2, 66, 600, 1, 32, "bool", torch.float16),
                                   (1, 64, 200, 2, 64, "add", torch.bfloat16), (1, 65, 322, 1, 64, "bool", torch.float16),
                                   (1, 9, 640, 2, 32, "add", torch.bfloat16)],
                          ids=lambda c: "-".join(str(x).replace("torch.", "") for x in c))
 def test_long_rows_sum_dbias_in_a_kernel_of_its_own(E, case):
-    """Rows of more than 384 keys (512 at head dims 8 and 16; 256 at head dim 32 with at most four
-    (batch, head) pairs; 128 at head dim 64) with at least 64 S rows (8 beyond 512 keys at head
-    dim 32): dQ from
+    """Rows of more than 512 keys (128 at head dim 64) that leave the last 256-key block of the
+    one-kernel form mostly empty, or for which it has no form, with at least 64 S rows (8 beyond
+    512 keys at head dim 32): dQ from
     the kernel whose waves own their query rows, the dBias partials from a second kernel that
     forms dS again (`evoattn_kernels` names both).  Against the CPU oracle in fp32, and against
     the one kernel that does both (EVO_FLAG_DEBUG_NO_DQ_SPLIT) to a 16-bit unit in the last place."""
