@@ -561,23 +561,25 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 // dO^T and Q^T fragments: row d = dt*32 + li, the 8 queries the P registers hold
-                const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                v8 gta = zero8<T>(), qta = zero8<T>();
-                if (col < D) {
+                // Lanes whose column lies past the head dim (rows d >= D of the fragments: rows of dK^T and
+                // dV^T that are never stored, and a row of the product depends on its own row of the A operand
+                // only) read column 0 instead of being masked and cleared for every tile.
+                const int col0 = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                const int col = (D % 32 == 0 || col0 < D) ? col0 : 0;
+                v8 gta, qta;
 #pragma unroll
-                    for (int h2 = 0; h2 < 2; ++h2) {
-                        const int row = qb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
-                        const int o = R::swz(row, col >> 3) + (col & 7) * 2;
-                        s16x4 rg = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (s16x4 __attribute__((address_space(3))) *)(lds + OFF_G + o));
-                        s16x4 rq = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (s16x4 __attribute__((address_space(3))) *)(lds + OFF_QR + o));
-                        v4 vg = __builtin_bit_cast(v4, rg), vq = __builtin_bit_cast(v4, rq);
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const int row = qb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                    const int o = R::swz(row, col >> 3) + (col & 7) * 2;
+                    s16x4 rg = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (s16x4 __attribute__((address_space(3))) *)(lds + OFF_G + o));
+                    s16x4 rq = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (s16x4 __attribute__((address_space(3))) *)(lds + OFF_QR + o));
+                    v4 vg = __builtin_bit_cast(v4, rg), vq = __builtin_bit_cast(v4, rq);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            gta[4 * h2 + i] = vg[i];
-                            qta[4 * h2 + i] = vq[i];
-                        }
+                    for (int i = 0; i < 4; ++i) {
+                        gta[4 * h2 + i] = vg[i];
+                        qta[4 * h2 + i] = vq[i];
                     }
                 }
                 dv[dt] = Mfma<T>::mma(gta, pf, dv[dt]);

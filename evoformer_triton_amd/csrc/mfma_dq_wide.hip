@@ -242,19 +242,20 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 // K^T fragment: row d = dt*32 + li, the 8 keys the dS registers hold
-                const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                v8 kta = zero8<T>();
-                if (col < D) {
+                // lanes whose column lies past the head dim (rows of the product that are never stored; a row of the
+                // product depends on its own row of this operand only) read column 0 instead of being masked and cleared
+                const int col0 = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                const int col = (D % 32 == 0 || col0 < D) ? col0 : 0;
+                v8 kta;
 #pragma unroll
-                    for (int h2 = 0; h2 < 2; ++h2) {
-                        const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
-                        const int o = R::swz(row, col >> 3) + (col & 7) * 2;
-                        s16x4w rk = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (s16x4w __attribute__((address_space(3))) *)(lds + R::OFF_K + o));
-                        v4 vk = __builtin_bit_cast(v4, rk);
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                    const int o = R::swz(row, col >> 3) + (col & 7) * 2;
+                    s16x4w rk = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (s16x4w __attribute__((address_space(3))) *)(lds + R::OFF_K + o));
+                    v4 vk = __builtin_bit_cast(v4, rk);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) kta[4 * h2 + i] = vk[i];
-                    }
+                    for (int i = 0; i < 4; ++i) kta[4 * h2 + i] = vk[i];
                 }
                 dqacc[dt] = Mfma<T>::mma(kta, dsf2[ts], dqacc[dt]);
             }

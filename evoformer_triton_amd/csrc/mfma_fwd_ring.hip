@@ -386,18 +386,19 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 for (int ts = 0; ts < 4; ++ts) {
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
-                        const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                        v8 va = zero8<T>();
-                        if (col < D) {
+                        // lanes whose column lies past the head dim (rows of the product that are never stored; a row of the
+                        // product depends on its own row of this operand only) read column 0 instead of being masked and cleared
+                        const int col0 = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+                        const int col = (D % 32 == 0 || col0 < D) ? col0 : 0;
+                        v8 va;
 #pragma unroll
-                            for (int h2 = 0; h2 < 2; ++h2) {
-                                const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
-                                const unsigned char *ad = buf + R::OFF_V + R::swz(row, col >> 3) + (col & 7) * 2;
-                                s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                    (s16x4 __attribute__((address_space(3))) *)ad);
-                                v4 rv = __builtin_bit_cast(v4, rd);
-                                va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
-                            }
+                        for (int h2 = 0; h2 < 2; ++h2) {
+                            const int row = kb + 16 * ts + 8 * h2 + 4 * g + ((lane & 15) >> 2);
+                            const unsigned char *ad = buf + R::OFF_V + R::swz(row, col >> 3) + (col & 7) * 2;
+                            s16x4 rd = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (s16x4 __attribute__((address_space(3))) *)ad);
+                            v4 rv = __builtin_bit_cast(v4, rd);
+                            va[4 * h2] = rv[0]; va[4 * h2 + 1] = rv[1]; va[4 * h2 + 2] = rv[2]; va[4 * h2 + 3] = rv[3];
                         }
                         oacc[dt] = Mfma<T>::mma(va, pf[ts], oacc[dt]);
                     }
