@@ -21,6 +21,11 @@ struct Geo {
     // the matrix core has k-steps to spare, its rounding residue is carried as well, which
     // makes the scores exact to fp32 (and identical in the forward and both backward kernels).
     static constexpr bool RESID = D <= 16;
+    // From head dim 16 on the extra columns have a k-step of their own (the last).  The operand
+    // that a wave keeps for a whole row holds zeros in that step's upper half (lane group 1), so
+    // the operand read per tile may hold any finite values there: both lane groups read the same
+    // extra columns, and no lane is cleared or masked per tile.
+    static __device__ __forceinline__ constexpr bool aug_step(int ks) { return !AUG_IN_PAD && ks == KS - 1; }
 };
 
 template <typename T>

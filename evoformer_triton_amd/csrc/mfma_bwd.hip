@@ -180,7 +180,7 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
                     if (d0 < D) {
                         ka[ks] = ld8(K + (int64_t)keyc * sn + d0);
                         va[ks] = ld8(V + (int64_t)keyc * sn + d0);
-                    } else if (d0 == AUGC) {
+                    } else if (d0 == AUGC || G::aug_step(ks)) {  // (qf, gf are zero in the step's upper half)
                         ka[ks] = aug8<T>(m2row[kb + li], one3);  // mask x ones, ones x -lse
                         va[ks] = aug8<T>(one3, zero3);           // ones x -delta
                     }
@@ -503,7 +503,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
                 const int o = R::swz(qb + li, 2 * ks + g);
                 qa = *reinterpret_cast<const v8 *>(lds + OFF_QS + o);
                 ga = *reinterpret_cast<const v8 *>(lds + OFF_G + o);
-            } else if (d0 == AUGC) {
+            } else if (d0 == AUGC || G::aug_step(ks)) {   // (kf, vf are zero in the step's upper half)
                 qa = *reinterpret_cast<const v8 *>(lds + OFF_AQ + (qb + li) * 16);
                 ga = *reinterpret_cast<const v8 *>(lds + OFF_AG + (qb + li) * 16);
             }

@@ -185,7 +185,7 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                             const int o = R::swz(kb + li, 2 * ks + g);
                             ka = *reinterpret_cast<const v8 *>(buf + R::OFF_K + o);
                             va = *reinterpret_cast<const v8 *>(buf + R::OFF_V + o);
-                        } else if (d0 == AUGC) {
+                        } else if (d0 == AUGC || G::aug_step(ks)) {   // (qf, gf are zero in the step's upper half)
                             ka = *reinterpret_cast<const v8 *>(buf + R::OFF_AK + (kb + li) * 16);
                             va = vaug;
                         }

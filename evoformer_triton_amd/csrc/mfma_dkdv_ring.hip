@@ -308,7 +308,7 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
                         const int o = R::swz(qb + li, 2 * ks + g);
                         qa = *reinterpret_cast<const v8 *>(buf + R::OFF_QS + o);
                         ga = *reinterpret_cast<const v8 *>(buf + R::OFF_G + o);
-                    } else if (d0 == AUGC) {
+                    } else if (d0 == AUGC || G::aug_step(ks)) {   // (kf, vf are zero in the step's upper half)
                         qa = *reinterpret_cast<const v8 *>(buf + R::OFF_AQ + (qb + li) * 16);
                         ga = *reinterpret_cast<const v8 *>(buf + R::OFF_AG + (qb + li) * 16);
                     }

@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
                 const int o = R::swz(kb + li, 2 * ks + g);
                 ka = *reinterpret_cast<const v8 *>(lds + R::OFF_K + o);
                 va = *reinterpret_cast<const v8 *>(lds + R::OFF_V + o);
-            } else if (d0 == AUGC) {
+            } else if (d0 == AUGC || G::aug_step(ks)) {   // (qf, gf are zero in the step's upper half)
                 ka = *reinterpret_cast<const v8 *>(lds + R::OFF_AK + (kb + li) * 16);
                 va = vaug;
             }
