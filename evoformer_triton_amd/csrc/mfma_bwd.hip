@@ -56,7 +56,8 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
     __shared__ __attribute__((aligned(16))) float red[4 * 32 * RP];
     __shared__ __attribute__((aligned(16))) T Kt[4 * DP * KTP];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it branches and is addressed by the scalar unit
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
@@ -362,7 +363,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
     EVO_TK(0);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it branches and is addressed by the scalar unit
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nkb = (p.N + BK - 1) / BK;
@@ -526,8 +528,10 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
         if (R::RESID) {
 #pragma unroll
             for (int ks = 0; ks < KSD; ++ks) {
-                v8 ql = zero8<T>();
-                if (ks * 16 + g * 8 < D) ql = *reinterpret_cast<const v8 *>(lds + OFF_QL + R::swz(qb + li, 2 * ks + g));
+                // (kres is zero in the lanes whose columns lie past the head dim: there this operand may hold
+                // any finite values, and those lanes read the row's first chunk rather than being cleared per tile)
+                const int ch = ks * 16 + g * 8 < D ? 2 * ks + g : 2 * ks;
+                const v8 ql = *reinterpret_cast<const v8 *>(lds + OFF_QL + R::swz(qb + li, ch));
                 acc = Mfma<T>::mma(ql, kres[ks], acc);
             }
         }

@@ -47,7 +47,8 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * R::LDS_BYTES];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it branches and is addressed by the scalar unit
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nqb = (p.N + R::QB - 1) / R::QB, nkb = (p.N + KB - 1) / KB;

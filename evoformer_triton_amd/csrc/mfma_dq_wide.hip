@@ -53,7 +53,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
 
     __shared__ __attribute__((aligned(1024))) unsigned char lds[R::LDS_BYTES];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it branches and is addressed by the scalar unit
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nqb = (p.N + BQ - 1) / BQ;

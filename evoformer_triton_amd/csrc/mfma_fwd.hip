@@ -71,7 +71,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
     __shared__ __attribute__((aligned(16))) T Ks[BKV * KP];
     __shared__ __attribute__((aligned(16))) T Vt[DP * VP];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // scalar: what depends on it branches and is addressed by the scalar unit
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
     const int nqb = (p.N + BQ - 1) / BQ;
