@@ -60,10 +60,10 @@ REDUCED = ("dBias", "dMask")    # sums of dS over S rows / over heads and querie
 
 
 def half_ulp(x, dtype):
-    """Half a unit in the last place of a 16-bit format at each |x|, from the entry's own binade:
-    the most that rounding a result to that format moves it."""
-    bits = {torch.bfloat16: 8, torch.float16: 11}[dtype]          # significand bits, the implicit one included
-    floor = 2.0 ** (-126 if dtype == torch.bfloat16 else -14)
+    """Half a unit in the last place of the format a result is stored in at each |x|, from the
+    entry's own binade: the most that rounding a result to that format moves it."""
+    bits = {torch.bfloat16: 8, torch.float16: 11, torch.float32: 24}[dtype]   # significand bits, the implicit one included
+    floor = 2.0 ** (-14 if dtype == torch.float16 else -126)
     return torch.exp2(torch.floor(torch.log2(x.abs().clamp_min(floor))) - bits)
 
 
