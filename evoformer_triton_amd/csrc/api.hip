@@ -333,7 +333,12 @@ const char *evoattn_path(const EvoAttnParams *p, int pass) {
 
 // rows of 129..256 keys: a workgroup per chunk of S rows with the head's bias resident
 static bool fwd_ring_ok(const EvoAttnParams &p) {
-    return !(p.flags & EVO_FLAG_PER_PROBLEM) && !bias_direct(p) && p.N > 128 && p.N <= mfma_fwdr_max_n(p.D);
+    if ((p.flags & EVO_FLAG_PER_PROBLEM) || bias_direct(p) || p.N <= 128 || p.N > mfma_fwdr_max_n(p.D)) return false;
+    // Resident, a bias in the dtype of q takes 64 registers, an fp32 bias 128, which fit the register file only at
+    // head dim 8 without a gate; elsewhere most of them are spilled and the one-workgroup-per-problem forward, which
+    // streams the tiles, serves an fp32 bias (B = 1, S = 512, N = 256, H = 8, D = 32: 130 against 214 us).
+    // EVO_FLAG_DEBUG_FWD_BIAS_TILES keeps the resident fp32 form, for comparison.
+    return !p.bias || p.bias_dtype == p.dtype || (p.D == 8 && !p.gate) || (p.flags & EVO_FLAG_DEBUG_FWD_BIAS_TILES);
 }
 
 // The dK/dV kernel that walks over a chunk of S rows keeps 16-bit bias columns resident: it

@@ -143,11 +143,20 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         const int bb = e.bias_batches > 1 ? b : 0;
         const T *brow = (const T *)p.bias + (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h +
                         (int64_t)qrow * p.bias_stride_row;
+        // rows that start on 16-byte boundaries are read in 16-byte pieces, others entry by entry (once per
+        // workgroup either way); uniform
+        const bool rows16 = p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 && p.bias_stride_b % 8 == 0 &&
+                            p.bias_stride_h % 8 == 0 && p.bias_stride_row % 8 == 0;
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
-            // chunks past the row repeat its last one (those keys carry the mask floor)
-            const int key0 = min((j >> 1) * 32 + 16 * (j & 1) + 8 * g, p.N - 8);
-            bres[j] = ld8(brow + key0);
+            // keys past the row repeat its last ones (they carry the mask floor)
+            const int key0 = (j >> 1) * 32 + 16 * (j & 1) + 8 * g;
+            if (rows16) {
+                bres[j] = ld8(brow + min(key0, p.N - 8));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) bres[j][i] = brow[min(key0 + i, p.N - 1)];
+            }
         }
     }
 
@@ -518,15 +527,21 @@ static int fwdr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     return p.gate ? fwdr_launch_g<T, D, BIASK, true>(p, e, st) : fwdr_launch_g<T, D, BIASK, false>(p, e, st);
 }
 
+// whether the form with resident fp32 bias tiles keeps them in registers (the dispatch in api.hip sends an
+// fp32 bias here under the same condition)
+static bool fwdr_tiles_fit(const EvoAttnParams &p) { return EVO_D == 8 && !p.gate; }
+
 template <typename T>
 static int fwdr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     if (p.bias_dtype == EVO_NONE) return fwdr_launch<T, EVO_D, 0>(p, e, st);
-    // The 16-bit form reads the caller's bias rows in 16-byte pieces; where it applies it is the
-    // faster one (64 resident registers instead of 128, no spills).  EVO_FLAG_DEBUG_FWD_BIAS_TILES selects
-    // the other form, for comparison.
-    const bool rows16 = p.bias_dtype == p.dtype && p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 &&
-                        p.bias_stride_b % 8 == 0 && p.bias_stride_h % 8 == 0 && p.bias_stride_row % 8 == 0;
-    return (rows16 && !(p.flags & EVO_FLAG_DEBUG_FWD_BIAS_TILES)) ? fwdr_launch<T, EVO_D, 2>(p, e, st) : fwdr_launch<T, EVO_D, 1>(p, e, st);
+    // Two resident forms.  fp32 tiles as C operands (128 registers) fit the register file only at head dim 8
+    // without a gate, and are the faster form there (S = 1024, N = 256, H = 8: 119 against 143 us; N = 201, S = 512:
+    // 64 against 85 us), also for an fp32 bias.  Elsewhere they spill 77..169 registers (head dim 16, N = 256: 170
+    // against 82 us) and a bias in the dtype of q stays resident as the caller's 16-bit rows (64 registers); an
+    // fp32 bias is then served by the one-workgroup-per-problem forward (the dispatch sends none here).
+    // EVO_FLAG_DEBUG_FWD_BIAS_TILES selects the fp32 tiles wherever the kernel runs, for comparison.
+    const bool tiles = fwdr_tiles_fit(p) || p.bias_dtype != p.dtype || (p.flags & EVO_FLAG_DEBUG_FWD_BIAS_TILES);
+    return tiles ? fwdr_launch<T, EVO_D, 1>(p, e, st) : fwdr_launch<T, EVO_D, 2>(p, e, st);
 }
 
 // Largest N this kernel takes for the head dim (0: not built for it).
