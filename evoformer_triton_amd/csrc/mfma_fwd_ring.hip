@@ -76,6 +76,16 @@ __device__ __forceinline__ float pair_sums(typename Mfma<T>::v8 x, float acc) {
     return dot8<T>(x, one, acc);
 }
 
+// The copy of a wave's 32 bias rows (256 keys, 16 bits each) that rows of unaligned length pass through: rows
+// 16 bytes further apart than their length, so that the 16-byte pieces of different rows fall into different banks.
+constexpr int kBiasCopyPitch = 256 * 2 + 16;
+constexpr int kBiasCopyBytes = 8 * 32 * kBiasCopyPitch;
+// whether every bias row starts on a 16-byte boundary and is a whole number of 16-byte pieces long
+static __host__ __device__ inline bool fwdr_rows16(const EvoAttnParams &p) {
+    return p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 && p.bias_stride_b % 8 == 0 && p.bias_stride_h % 8 == 0 &&
+           p.bias_stride_row % 8 == 0;
+}
+
 // BIASK: 0 no bias, 1 fp32 tiles (x log2(e), accumulator order) as C operands, 2 the caller's 16-bit rows through the identity
 // GATED: the output gate in the epilogue (a kernel of its own: the ungated one carries none of its registers)
 template <typename T, int D, int BIASK, bool GATED>
@@ -143,20 +153,40 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         const int bb = e.bias_batches > 1 ? b : 0;
         const T *brow = (const T *)p.bias + (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h +
                         (int64_t)qrow * p.bias_stride_row;
-        // rows that start on 16-byte boundaries are read in 16-byte pieces, others entry by entry (once per
-        // workgroup either way); uniform
-        const bool rows16 = p.N % 8 == 0 && ((uintptr_t)p.bias & 15) == 0 && p.bias_stride_b % 8 == 0 &&
-                            p.bias_stride_h % 8 == 0 && p.bias_stride_row % 8 == 0;
+        // Rows that start on 16-byte boundaries are read in 16-byte pieces.  Other rows (a row length that is no
+        // multiple of 8) go through LDS once per workgroup: every wave copies its 32 rows with the lanes along the
+        // row (coalesced 2-byte loads; a lane per row would touch 64 cache lines per load) and takes its pieces from
+        // there.  The copy lies where the stages will (and beyond: the launcher asks for kBiasCopyBytes of LDS for
+        // such rows), so a barrier separates the last read from the first stage.
+        const bool rows16 = fwdr_rows16(p);   // uniform
+        if (rows16) {
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            // keys past the row repeat its last ones (they carry the mask floor)
-            const int key0 = (j >> 1) * 32 + 16 * (j & 1) + 8 * g;
-            if (rows16) {
+            for (int j = 0; j < 16; ++j) {
+                // chunks past the row repeat its last one (those keys carry the mask floor)
+                const int key0 = (j >> 1) * 32 + 16 * (j & 1) + 8 * g;
                 bres[j] = ld8(brow + min(key0, p.N - 8));
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) bres[j][i] = brow[min(key0 + i, p.N - 1)];
             }
+        } else {
+            unsigned char *wb = lds + wave * (32 * kBiasCopyPitch);
+            const T *bmat = (const T *)p.bias + (int64_t)bb * p.bias_stride_b + (int64_t)h * p.bias_stride_h;
+            for (int r = 0; r < 32; ++r) {
+                const T *row = bmat + (int64_t)min(q0 + r, p.N - 1) * p.bias_stride_row;
+#pragma unroll
+                for (int cc = 0; cc < 4; ++cc) {
+                    const int key = cc * 64 + lane;   // keys past the row repeat its last one
+                    *reinterpret_cast<T *>(wb + r * kBiasCopyPitch + key * 2) = row[min(key, p.N - 1)];
+                }
+            }
+            // (LDS serves a wave's accesses in order; the fence keeps the compiler from moving the reads up)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int key0 = (j >> 1) * 32 + 16 * (j & 1) + 8 * g;
+                bres[j] = *reinterpret_cast<const v8 *>(wb + li * kBiasCopyPitch + key0 * 2);
+            }
+            __syncthreads();
         }
     }
 
@@ -510,14 +540,16 @@ static int fwdr_launch_g(const EvoAttnParams &p, const Extra &e0, hipStream_t st
     static PerDevice done{};
     int cus = 256;
     auto kern = mfma_fwd_ring<T, D, BIASK, GATED>;
-    if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, &cus)) return rc;
+    constexpr int LDS_MOST = BIASK == 2 && R::LDS_BYTES < kBiasCopyBytes ? kBiasCopyBytes : R::LDS_BYTES;
+    if (const int rc = ensure_dynamic_lds((const void *)kern, LDS_MOST, done, &cus)) return rc;
+    const int lds_bytes = BIASK == 2 && !fwdr_rows16(p) ? LDS_MOST : R::LDS_BYTES;
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     Extra e = e0;
     const int bh = p.B * p.H;
     const int want = chunks_for_rounds(bh, p.S, cus, 0.0);
     e.chunk = (p.S + want - 1) / want;
     e.n_chunks = (p.S + e.chunk - 1) / e.chunk;
-    kern<<<(unsigned)bh * (unsigned)e.n_chunks, 512, R::LDS_BYTES, st>>>(p, e);
+    kern<<<(unsigned)bh * (unsigned)e.n_chunks, 512, lds_bytes, st>>>(p, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }

@@ -278,7 +278,7 @@ SMALL = [
     (1, 40, 256, 1, 32, "add", "q", "ds4sci"),
     (1, 9, 192, 2, 32, None, None, "reference"),
     (2, 6, 256, 3, 32, "add", "q", "ds4sci"),          # per-head strides, bias per batch entry
-    (1, 5, 252, 2, 32, "bool", "q", "reference"),      # bias rows not 16-byte aligned: read entry by entry
+    (1, 5, 252, 2, 32, "bool", "q", "reference"),      # bias rows not 16-byte aligned: copied through LDS
     (1, 5, 256, 2, 16, "soft", torch.float32, "reference"),
     (2, 3, 136, 2, 8, "add", "q", "reference"),
     (1, 5, 200, 2, 32, "soft", "q", "reference"),      # dMask partials from the chunk-of-rows dK/dV
