@@ -123,13 +123,19 @@ static bool dq_wide_grid_ok(const EvoAttnParams &p) {
 // N = 704 2.01 / 2.06 ms.
 // EVO_FLAG_DEBUG_NO_DQ_SPLIT selects the one kernel, for comparison.
 static bool dq_split_ok(const EvoAttnParams &p) {
-    // fewest S rows: the second kernel's start-up has to pay (N = 768, D = 32: ahead from 8 rows on)
-    const int min_s = p.N > 2048 ? 2 : p.D == 32 && p.N > 512 ? 8 : 64;   // (beyond 2048 keys the one kernel has no form at all)
     const int min_n = p.D == 64 ? 128 : 512;
     if (p.D > 64) return false;   // the dBias kernel is not built for head dim 128
     const int rem = p.N % 256;
     const bool full_blocks = rem == 0 || rem >= (p.D == 32 ? 224 : 192);
-    if (full_blocks && dq_ring_ok(p)) return false;
+    const bool ring = dq_ring_ok(p);
+    if (full_blocks && ring) return false;
+    // Fewest S rows: the second kernel's start-up has to pay.  Against the one kernel over a chunk of rows
+    // (N = 768, D = 32: ahead from 8 rows on); where that kernel has no form, against the one-workgroup-per-problem
+    // dQ kernel, which the pair beats from 8 rows on (bf16, dQ + dBias, us, S = 8 / 16 / 32 / 52: D = 8, H = 8, N = 768
+    // 50 / 71 / 102 / 146 against 47 / 92 / 159 / 228; D = 16, N = 1024, S = 8 / 16 / 32: 53 / 84 / 152 against
+    // 63 / 99 / 175; D = 64, H = 4, N = 1024, S = 16 / 32 / 59: 99 / 194 / 327 against 152 / 277 / 599; N = 300,
+    // S = 16 / 32: 32 / 41 against 30 / 47).  Beyond 2048 keys that kernel has no form either.
+    const int min_s = p.N > 2048 ? 2 : !ring ? (p.D == 64 ? 16 : 8) : p.D == 32 && p.N > 512 ? 8 : 64;
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
 }
