@@ -137,7 +137,7 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     // S = 16 / 32: 32 / 41 against 30 / 47).  Beyond 2048 keys that kernel has no form either.
     const int min_s = p.N > 2048 ? 2 : !ring ? (p.D == 64 ? 16 : 8) : p.D == 32 && p.N > 512 ? 8 : 64;
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
-    return p.bias_dtype == p.dtype;   // it keeps the bias tiles as 16-bit pairs
+    return p.bias_dtype == p.dtype || p.bias_dtype == EVO_F32;   // (the dBias kernel keeps 16-bit pairs or fp32 tiles)
 }
 
 static bool dq_wide_ok(const EvoAttnParams &p) {

@@ -36,7 +36,9 @@ struct DbGeo {
     static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
 };
 
-template <typename T, int D>
+// BF32: the bias is fp32 (its prepared tiles are fp32 in log2 units and stay resident as they are: twice the
+// registers of the 16-bit pairs, nothing to unpack)
+template <typename T, int D, bool BF32>
 __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef DbGeo<D> R;
@@ -73,15 +75,25 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
     // use they are unpacked and multiplied by log2(e) in fp32, the product the fp32 tiles hold.
     const int bb = e.bias_batches > 1 ? b : 0;
     const int qtc = min(q0 >> 5, NT - 1);
-    unsigned bres[TPW][8];
+    unsigned bres[BF32 ? 1 : TPW][8];
+    f32x16 bres32[BF32 ? TPW : 1];
     f32x16 dbacc[TPW];
 #pragma unroll
     for (int j = 0; j < TPW; ++j) {
         const int kt = min(k0 / 32 + j, NT - 1);
-        Tile16 t;
-        load_tile16(e.bq16 + ((((int64_t)bb * p.H + h) * NT + qtc) * NT + kt) * 1024 + lane * 16, t);
+        const int64_t o = ((((int64_t)bb * p.H + h) * NT + qtc) * NT + kt) * 1024 + lane * 16;
+        if constexpr (BF32) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) bres[j][i] = t.w[i >> 2][i & 3];
+            for (int rr = 0; rr < 4; ++rr) {
+                const f32x4 v = *reinterpret_cast<const f32x4 *>(e.bq + o + 4 * rr);
+                bres32[j][4 * rr] = v[0]; bres32[j][4 * rr + 1] = v[1]; bres32[j][4 * rr + 2] = v[2]; bres32[j][4 * rr + 3] = v[3];
+            }
+        } else {
+            Tile16 t;
+            load_tile16(e.bq16 + o, t);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) bres[j][i] = t.w[i >> 2][i & 3];
+        }
 #pragma unroll
         for (int r = 0; r < 16; ++r) dbacc[j][r] = 0.0f;
     }
@@ -165,16 +177,21 @@ __global__ void __launch_bounds__(256, 2) mfma_dbias(EvoAttnParams p, Extra e) {
                 if (j < nt) {   // uniform
                     const int kb = j * 32;
                     f32x16 acc, dp;
+                    if constexpr (BF32) {
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        // unpack per use: expanded once and for all the tiles would take twice the
-                        // registers (the empty statement "changes" the resident register in place, so
-                        // that its expansion cannot be moved out of the loop over S, at no copy)
-                        asm volatile("" : "+v"(bres[j][i]));
-                        float lo, hi;
-                        unpack2<T>(bres[j][i], lo, hi);
-                        acc[2 * i] = lo * bscale;
-                        acc[2 * i + 1] = hi * bscale;
+                        for (int r = 0; r < 16; ++r) acc[r] = dead ? 0.0f : bres32[j][r];   // (uniform)
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            // unpack per use: expanded once and for all the tiles would take twice the
+                            // registers (the empty statement "changes" the resident register in place, so
+                            // that its expansion cannot be moved out of the loop over S, at no copy)
+                            asm volatile("" : "+v"(bres[j][i]));
+                            float lo, hi;
+                            unpack2<T>(bres[j][i], lo, hi);
+                            acc[2 * i] = lo * bscale;
+                            acc[2 * i + 1] = hi * bscale;
+                        }
                     }
 #pragma unroll
                     for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
@@ -246,8 +263,14 @@ int64_t EVO_CAT(mfma_dbias_blocks_d, EVO_D)(const EvoAttnParams &p) {
 int EVO_CAT(launch_mfma_dbias_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     const int64_t grid = EVO_CAT(mfma_dbias_blocks_d, EVO_D)(p) * e.n_chunks;
     if (grid <= 0 || grid > 0x7fffffff) return EVO_EOVERFLOW;
-    if (p.dtype == EVO_BF16) mfma_dbias<bf16_t, EVO_D><<<(unsigned)grid, 256, 0, st>>>(p, e);
-    else mfma_dbias<f16_t, EVO_D><<<(unsigned)grid, 256, 0, st>>>(p, e);
+    const bool bf32 = p.bias_dtype == EVO_F32;
+    if (p.dtype == EVO_BF16) {
+        if (bf32) mfma_dbias<bf16_t, EVO_D, true><<<(unsigned)grid, 256, 0, st>>>(p, e);
+        else mfma_dbias<bf16_t, EVO_D, false><<<(unsigned)grid, 256, 0, st>>>(p, e);
+    } else {
+        if (bf32) mfma_dbias<f16_t, EVO_D, true><<<(unsigned)grid, 256, 0, st>>>(p, e);
+        else mfma_dbias<f16_t, EVO_D, false><<<(unsigned)grid, 256, 0, st>>>(p, e);
+    }
     return hip_rc();
 }
 

@@ -616,7 +616,7 @@ LONG_ROWS = [  # B, S, N, H, D, mask, bias dtype, dBias asked for, backward on t
     (1, 1, 2304, 2, 64, "add", "q", True, True),               # S = 1: dBias written by the dQ kernel
     (1, 2, 2560, 1, 16, "bool", None, False, True),            # no bias
     (1, 3, 2304, 1, 32, "soft", torch.float32, False, True),   # bias as a constant
-    (1, 2, 2304, 1, 32, "bool", torch.float32, True, False),   # fp32 bias with a gradient: the plain kernels
+    (1, 2, 2304, 1, 32, "bool", torch.float32, True, True),    # fp32 bias with a gradient: the dBias kernel with fp32 tiles
 ]
 
 
