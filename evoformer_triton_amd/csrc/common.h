@@ -103,6 +103,20 @@ __device__ __forceinline__ Prob decode_problem(const EvoAttnParams &p, unsigned 
     return r;
 }
 
+// The t-th problem in the order the one-workgroup-per-problem kernels walk them (consecutive t run on one XCD,
+// behind one L2).  Where the heads lie inside a token (the per-head layout) and a head's row is shorter than a
+// cache line, the line holds rows of several heads, and the heads of one (b, s) follow each other (bf16, forward /
+// dK/dV in that layout: C5, 8 heads to a line, 335 -> 295 / 480 -> 405 us; C3, two to a line, 98 -> 94 / 127 ->
+// 116 us; at C4's 768 keys 597 -> 608 / 770 -> 768 us, and head dim 64 loses 2 %: there and elsewhere a head's S
+// rows follow each other).
+__device__ __forceinline__ Prob walk_problem(const EvoAttnParams &p, unsigned t) {
+    if (p.stride_h < p.stride_n && (p.D <= 16 || (p.D == 32 && p.N <= 512))) {
+        const unsigned h = t % p.H, bs = t / p.H;
+        return decode_problem(p, ((bs / p.S) * p.H + h) * p.S + bs % p.S);
+    }
+    return decode_problem(p, t);
+}
+
 // Additive form of mask[b][s][key]; -inf past the end of the row so that padded keys get
 // zero probability whatever the rest of the row holds.
 __device__ __forceinline__ float mask_add(const EvoAttnParams &p, int b, int s, int key) {

@@ -339,8 +339,19 @@ __global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_
     if (i >= pieces) return;
     const int c = (int)(i % cpr);
     const int64_t r = i / cpr;
-    const Prob pr = decode_problem(p, (unsigned)(r / p.N));
-    const int64_t off = pr.base + (r % p.N) * p.stride_n + c * 8;
+    int64_t off;
+    if (p.stride_h < p.stride_n) {
+        // heads inside a token (the per-head layout): rows in the order they lie in memory, (b, s, n, h), so that
+        // a wave's pieces are neighbours (in problem order they are one head's 16 D bytes out of every token)
+        const int h = (int)(r % p.H);
+        const int64_t tok = r / p.H;
+        const int n = (int)(tok % p.N);
+        const int64_t bs = tok / p.N;
+        off = (bs / p.S) * p.stride_b + (bs % p.S) * p.stride_s + (int64_t)n * p.stride_n + (int64_t)h * p.stride_h + c * 8;
+    } else {
+        const Prob pr = decode_problem(p, (unsigned)(r / p.N));
+        off = pr.base + (r % p.N) * p.stride_n + c * 8;
+    }
     const T *go = (const T *)p.dout + off, *gl = (const T *)p.gate + off, *o = (const T *)p.o + off;
     T *d_o = dout_ungated + off, *d_g = (T *)p.dgate + off;
     // eight elements at a time: 16-byte loads and stores for the 16-bit types (the pieces are

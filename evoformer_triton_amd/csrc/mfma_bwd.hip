@@ -375,7 +375,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nkb;
     const int key0 = (lid % nkb) * BK + wave * 32;
-    const Prob pr = decode_problem(p, pid);
+    const Prob pr = walk_problem(p, pid);
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
     const T *Gd = (const T *)p.dout + pr.base;
     const int64_t sn = p.stride_n;

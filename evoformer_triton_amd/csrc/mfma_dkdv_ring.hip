@@ -67,8 +67,11 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, g = lane >> 5;
     const int NT = (p.N + 31) / 32, npad = NT * 32;
-    const unsigned bh = blockIdx.x % (unsigned)(p.B * p.H);
-    const int c = blockIdx.x / (unsigned)(p.B * p.H);
+    // Where the heads lie inside a token (the per-head layout) a cache line holds rows of several heads: the heads
+    // of a chunk of S rows then run on one XCD, behind one L2 (consecutive workgroup ids go round the XCDs).
+    const unsigned wid = p.stride_h < p.stride_n ? xcd_remap(blockIdx.x, gridDim.x) : blockIdx.x;
+    const unsigned bh = wid % (unsigned)(p.B * p.H);
+    const int c = wid / (unsigned)(p.B * p.H);
     const int b = bh / p.H, h = bh % p.H;
     const int key0 = wave * 32;
     const bool active = key0 < p.N;           // wave-uniform

@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
     const unsigned lid = xcd_remap(blockIdx.x, gridDim.x);
     const unsigned pid = lid / nqb;
     const int q0 = (lid % nqb) * BQ + wave * 32;
-    const Prob pr = decode_problem(p, pid);
+    const Prob pr = walk_problem(p, pid);
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
     const T *Gd = (const T *)p.dout + pr.base, *O = (const T *)p.o + pr.base;
     const int64_t sn = p.stride_n;
