@@ -124,8 +124,34 @@ def _alloc_bytes(nbytes, device):
     return torch.empty((max(int(nbytes), 256),), device=device, dtype=torch.uint8)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device):
+    """The current stream of `device` as the pointer the C ABI takes (the raw handle where torch
+    offers it: building a Stream object per call costs the host ten microseconds)."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(device.index if device.index is not None else torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+class _on_device:
+    """`torch.cuda.device(device)` where the current device is another one, nothing otherwise
+    (entering and leaving the guard costs the host more than the rest of a small call)."""
+
+    def __init__(self, device):
+        self.guard = None
+        if device.index is not None and device.index != torch.cuda.current_device():
+            self.guard = torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
 
 
 def _check_qkv(Q, K, V):
@@ -175,7 +201,7 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False, gate=None)
     Qp, Kp, Vp = _padded(Qc, Dp), _padded(Kc, Dp), _padded(Vc, Dp)
     mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
     bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
-    with torch.cuda.device(Q.device):
+    with _on_device(Q.device):
         O = torch.empty_like(Qp)                               # evoformer.py:654
         lse = torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32)   # :669-671
         p = _params(Qp, Kp, Vp, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
@@ -238,7 +264,7 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
         gate = None if gate is None else _padded(gate, Dp)
     want_dbias = bool(need_dbias and bias is not None)
     want_dmask = bool(need_dmask and mask is not None and mask.is_floating_point())
-    with torch.cuda.device(Q.device):
+    with _on_device(Q.device):
         dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)   # :749-751
         p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
         p.dout, p.dq, p.dk, p.dv = _ptr(dO), _ptr(dQ), _ptr(dK), _ptr(dV)

@@ -123,10 +123,15 @@ def test_path_selection(lib):
     assert lib.evoattn_path(ctypes.byref(p), 0) == b"generic"
     p = good(N=4096)
     assert lib.evoattn_path(ctypes.byref(p), 0) == b"mfma"
-    assert lib.evoattn_path(ctypes.byref(p), 1) == b"generic"            # dBias tiles exceed the register file
-    p.bias_dtype = p.dbias_dtype = _lib.EVO_BF16                           # ... unless a kernel of its own sums dBias
+    # the dBias sums of so long a row exceed the register file of the dQ kernels: a kernel of its own sums dBias,
+    # for a bias in fp32 and in the dtype of q alike
     assert lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
     assert lib.evoattn_kernels(ctypes.byref(p), 1) == b"mfma_dq_wide+mfma_dbias,mfma_dkdv"
+    p.bias_dtype = p.dbias_dtype = _lib.EVO_BF16
+    assert lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
+    assert lib.evoattn_kernels(ctypes.byref(p), 1) == b"mfma_dq_wide+mfma_dbias,mfma_dkdv"
+    p = good(N=4096, D=128)                                                # (that kernel is not built for head dim 128)
+    assert lib.evoattn_path(ctypes.byref(p), 1) == b"generic"
     p = good(N=4096)
     p.dbias = None
     assert lib.evoattn_path(ctypes.byref(p), 1) == b"mfma"
