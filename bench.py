@@ -70,6 +70,9 @@ def parse():
                          "B=4, H=32, D=64, N_seq=1, bool mask, fp32 pair bias, modes fwd / bwd / full, timed like "
                          "triton.testing.do_bench with the caches flushed before every repetition) on this build; "
                          "prints one JSON line with TFLOP/s per N beside the numbers the reference publishes")
+    ap.add_argument("--shape-sweep", action="store_true",
+                    help="forward and backward times over row lengths, head dims, bias dtypes and both layouts, and "
+                         "over the reference's own test shapes (test.py:82-100), as one JSON line")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy three times: under rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
@@ -165,6 +168,69 @@ def reference_sweep():
                                           "peak_memory_bf16_bias": mem}}))
 
 
+def shape_sweep():
+    """Forward and backward of `evoformer_attention` (autograd path, bf16, bool mask) over shapes either side of the
+    row lengths and head dims at which the library changes kernels, with a bias in the dtype of q, in fp32 and without,
+    in both layouts; then the reference's own test matrix (test.py:82-100: fp32 bias, head dim 64).  Rates are in
+    10^12 scores per second (B*H*S*N^2 scores per pass), which compares shapes of one head dim directly."""
+    import torch
+    from evoformer_triton_amd import evoformer_attention
+    dev = torch.device("cuda:0")
+
+    def timeit(fn, n=20):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(6):
+            fn()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e3
+
+    def one(B, S, N, H, D, bias_kind, layout):
+        g = torch.Generator(device=dev).manual_seed(1)
+        q, k, v, dO = (torch.randn((B, S, N, H, D), device=dev, generator=g).to(torch.bfloat16) for _ in range(4))
+        q, k, v = (t.requires_grad_() for t in (q, k, v))
+        mask = torch.rand((B, S, 1, 1, N), device=dev, generator=g) < 0.9
+        bias = None
+        if bias_kind != "none":
+            bias = (torch.randn((B, 1, H, N, N), device=dev, generator=g) * 0.5)
+            bias = bias.to(torch.bfloat16 if bias_kind == "q" else torch.float32).requires_grad_()
+        o = evoformer_attention(q, k, v, mask, bias, layout=layout)
+
+        def bwd():
+            q.grad = k.grad = v.grad = None
+            if bias is not None:
+                bias.grad = None
+            o.backward(dO, retain_graph=True)
+
+        tf = timeit(lambda: evoformer_attention(q, k, v, mask, bias, layout=layout))
+        tb = timeit(bwd)
+        sc = B * H * S * N * N / 1e6
+        return {"shape": [B, S, N, H, D], "bias": bias_kind, "layout": layout, "fwd_us": round(tf, 1), "bwd_us": round(tb, 1),
+                "fwd_rate": round(sc / tf, 2), "bwd_rate": round(sc / tb, 2)}
+
+    t_end = time.perf_counter() + 1.0                      # the chip needs a moment of load to reach its clocks
+    while time.perf_counter() < t_end:
+        one(1, 128, 256, 8, 32, "q", "reference")
+    rows = []
+    for D in (8, 16, 32, 64):
+        for N in (128, 200, 251, 256, 257, 384, 512, 640, 768, 1024, 2048):
+            H = 8 if D <= 32 else 4
+            S = max(2, min(1024, int(2.5e8 / (H * N * N))))
+            for bias_kind in ("q", "fp32", "none"):
+                rows.append(one(1, S, N, H, D, bias_kind, "reference"))
+            rows.append(one(1, S, N, H, D, "q", "ds4sci"))
+    ref = []
+    for (B, H, S, N, D) in ((1, 16, 1, 128, 64), (1, 4, 128, 128, 32), (5, 10, 200, 384, 64), (10, 5, 200, 384, 64),
+                            (1, 10, 200, 640, 64), (1, 15, 200, 640, 64), (1, 5, 100, 768, 64), (1, 10, 100, 768, 64),
+                            (1, 1, 100, 1280, 64), (1, 5, 300, 512, 64), (1, 5, 300, 384, 64)):
+        ref.append(one(B, S, N, H, D, "fp32", "reference"))
+    print(json.dumps({"shape_sweep": {"unit": "us; rates in 1e12 scores/s", "rows": rows, "reference_test_shapes": ref}}))
+
+
 def cpu_baseline(cfg, shape, budget_s=15.0, with_bias=True):
     """The eager oracle (fp32, chunked over S) on the host cores, on a slice of S rows."""
     import torch
@@ -197,6 +263,8 @@ def main():
         sys.exit(2)
     if args.reference_sweep:
         return reference_sweep()
+    if args.shape_sweep:
+        return shape_sweep()
     import torch
     from oracle import eager
     import evoformer_triton_amd.evoformer as E
