@@ -218,8 +218,10 @@ static PrepLayout prep_layout(const EvoAttnParams &p) {
         w.bq16 = off; off += align_up(tile_elems * 2);
         w.bk16 = off; off += align_up(tile_elems * 2);
     }
-    // transposed 16-bit copy for the kernels that keep bias columns resident
-    const bool bt_ok = p.bias && !bias_direct(p) && p.bias_dtype == p.dtype && p.N % 8 == 0;
+    // transposed 16-bit copy for the kernel that keeps bias columns resident (the chunk-of-rows dK/dV: rows of
+    // 129 keys up to its longest)
+    const bool bt_ok = p.bias && !bias_direct(p) && p.bias_dtype == p.dtype && p.N % 8 == 0 && p.N > 128 &&
+                       p.N <= mfma_kvr_max_n(p.D);
     w.bt = bt_ok ? off : (size_t)-1;
     if (bt_ok) off += align_up((size_t)w.bias_batches * p.H * p.N * p.N * 2);
     w.m2 = off; off += align_up((size_t)p.B * p.S * NT * 32 * 8);
