@@ -87,6 +87,14 @@ static int bias_vec_ok(const EvoAttnParams &p) {
 // allow 16-byte (fp32) or 8-byte loads.  EVO_FLAG_DEBUG_BIAS_TILES keeps the tiles, for comparison.
 static bool bias_direct(const EvoAttnParams &p) {
     if (!p.bias || p.S > 4 || (p.flags & EVO_FLAG_DEBUG_BIAS_TILES) || p.N % 4) return false;
+    // The 16-bit tiles of a bias in the dtype of q are cheap to prepare (2 + 4 bytes of traffic per entry at
+    // streaming rate) and pay from the first S row on where the score work per entry is small: they are taken
+    // for rows beyond 256 keys unless S = 1 at head dim 64 or more (whole step, us, tiles against the caller's
+    // tensor: H = 8, D = 32, N = 1024, S = 1 / 2 / 4 103 / 111 / 151 against 121 / 142 / 189; N = 2048 210 / 357 / 444
+    // against 244 / 418 / 545; B = 4, H = 32, D = 64, N = 1024, S = 1 / 2 / 4 596 / 1383 / 2320 against 536 / 1528 /
+    // 2718; up to 256 keys the tiles would bring the chunk-of-rows kernels, which need more S rows: 49 against
+    // 40 us at S = 4).  An fp32 bias keeps the direct reads up to 4 rows (S = 1: 257 against 140 us).
+    if (p.bias_dtype == p.dtype && p.dtype != EVO_F32 && p.N > 256 && !(p.S == 1 && p.D >= 64)) return false;
     // beyond 2048 keys a dBias summed over several S rows needs the kernel that reads prepared tiles
     // (decided without looking at dbias: the forward, which prepares, has none)
     if (p.N > 2048 && p.S > 1) return false;
