@@ -142,12 +142,12 @@ static bool dq_split_ok(const EvoAttnParams &p) {
     // dQ kernel, which the pair beats from 8 rows on (bf16, dQ + dBias, us, S = 8 / 16 / 32 / 52: D = 8, H = 8, N = 768
     // 50 / 71 / 102 / 146 against 47 / 92 / 159 / 228; D = 16, N = 1024, S = 8 / 16 / 32: 53 / 84 / 152 against
     // 63 / 99 / 175; D = 64, H = 4, N = 1024, S = 16 / 32 / 59: 99 / 194 / 327 against 152 / 277 / 599; N = 300,
-    // S = 16 / 32: 32 / 41 against 30 / 47), and from 1024 keys on from the first S count that does not read the
-    // caller's bias directly (whole step, us, the pair against that kernel: D = 32, H = 8, N = 1024, S = 5 / 7
-    // 149 / 159 against 185 / 215; N = 2048, S = 7 600 against 826; D = 8 472 against 730; D = 64, H = 4, S = 12
-    // 619 against 843; at N = 640..768 with S = 5, 6 the one kernel stays ahead, 76 / 103 against 88 / 111).
-    // Beyond 2048 keys that kernel has no form either.
-    const int min_s = p.N > 2048 ? 2 : !ring ? (p.N >= 1024 ? 5 : p.D == 64 ? 16 : 8) : p.D == 32 && p.N > 512 ? 8 : 64;
+    // S = 16 / 32: 32 / 41 against 30 / 47), and from 1024 keys on from 2 rows (whole step, us, the pair against
+    // that kernel: D = 32, H = 8, N = 1024, S = 2 / 3 / 4 / 5 / 7 108 / 113 / 114 / 149 / 159 against 110 / 131 / 150 /
+    // 185 / 215; N = 2048, S = 4 / 7 331 / 600 against 444 / 826; D = 8, S = 7 472 against 730; D = 64, B = 4, H = 32,
+    // N = 1024, S = 4 1.89 against 2.33 ms; at N = 640..768 with S = 5, 6 the one kernel stays ahead, 76 / 103
+    // against 88 / 111).  Beyond 2048 keys that kernel has no form either.
+    const int min_s = p.N >= 1024 ? 2 : !ring ? (p.D == 64 ? 16 : 8) : p.D == 32 && p.N > 512 ? 8 : 64;
     if (!p.dbias || p.S < min_s || p.N <= min_n || (p.flags & EVO_FLAG_DEBUG_NO_DQ_SPLIT) || bias_direct(p) || !dq_wide_grid_ok(p)) return false;
     return p.bias_dtype == p.dtype || p.bias_dtype == EVO_F32;   // (the dBias kernel keeps 16-bit pairs or fp32 tiles)
 }
