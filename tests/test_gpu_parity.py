@@ -249,6 +249,50 @@ def test_c_abi_under_graph_capture(E):
             assert torch.equal(a, b), rep
 
 
+@pytest.mark.parametrize("shape,gated", [((1, 16, 64, 4, 32), False), ((1, 64, 256, 8, 32), False),
+                                         ((1, 32, 384, 4, 32), False), ((1, 16, 128, 4, 32), True),
+                                         ((1, 1, 512, 4, 64), False)])
+def test_autograd_step_under_graph_capture(E, shape, gated):
+    """A whole step through the public function and autograd (forward, every gradient, the torch allocator's
+    buffers) captured with torch.cuda.graph: the host side allocates through torch only, reads nothing back
+    and launches on the current stream, so replays, with fresh inputs and eager steps between them, give bit
+    for bit what the eager step gives.  (Small steps are bound by the host: a replay is one launch.)"""
+    B, S, N, H, D = shape
+    dev = "cuda"
+    g = torch.Generator().manual_seed(5)
+    mk = lambda *s: torch.randn(s, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, dO = (mk(*shape) for _ in range(4))
+    bias = mk(1, 1, H, N, N) * 0.5
+    gate = mk(*shape) if gated else None
+    mask = torch.where(torch.rand((B, S, 1, 1, N), generator=g) < 0.9, 0.0, -1e9).to(torch.bfloat16).to(dev)
+    leaves = [q, k, v, bias] + ([gate] if gated else [])
+    for t in leaves:
+        t.requires_grad_()
+
+    def step():
+        o = E.evoformer_attention(q, k, v, mask, bias, gate=gate)
+        return (o,) + tuple(torch.autograd.grad(o, leaves, dO))
+
+    step()                                    # first use of the kernels outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for rep in range(3):
+        with torch.no_grad():
+            for t in [q, k, v, dO] + ([gate] if gated else []):
+                t.copy_(torch.randn(t.shape, generator=g).to(torch.bfloat16))
+            bias.copy_((torch.randn(bias.shape, generator=g) * 0.5).to(torch.bfloat16))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()                         # eager work between the replays
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.isfinite(b.float()).all()
+            assert torch.equal(a, b), (rep, i)
+
+
 # ------------------------------------------------------------------ small seeded cases vs the CPU oracle
 
 SMALL = [
