@@ -252,6 +252,7 @@ def test_c_abi_under_graph_capture(E):
 @pytest.mark.parametrize("shape,gated", [((1, 16, 64, 4, 32), False), ((1, 64, 256, 8, 32), False),
                                          ((1, 32, 384, 4, 32), False), ((1, 16, 128, 4, 32), True),
                                          ((1, 1, 512, 4, 64), False)])
+@pytest.mark.filterwarnings("ignore:The AccumulateGrad node's stream")   # the capture runs on a stream of its own
 def test_autograd_step_under_graph_capture(E, shape, gated):
     """A whole step through the public function and autograd (forward, every gradient, the torch allocator's
     buffers) captured with torch.cuda.graph: the host side allocates through torch only, reads nothing back
