@@ -97,3 +97,42 @@ def test_block_operands_are_views_of_the_projections():
         assert t.is_contiguous() and tuple(t.shape) == (1, 3, 40, 2, 16)
     assert tuple(bias.shape) == (1, 1, 2, 40, 40) and bias.dtype == torch.bfloat16 and bias.is_contiguous()
     assert tuple(add_mask.shape) == (1, 3, 1, 1, 40) and float(add_mask.abs().max()) == 0.0
+
+
+@pytest.mark.filterwarnings("ignore:The AccumulateGrad node's stream")   # the capture runs on a stream of its own
+@pytest.mark.parametrize("case", [(1, 12, 256, 4, 32, 64, 32), (2, 5, 100, 2, 16, 32, 16)], ids=lambda c: "-".join(map(str, c)))
+def test_block_step_under_graph_capture(case):
+    """The whole block, forward and every gradient (library GEMMs, LayerNorm, the kernels), captured with
+    torch.cuda.graph: replays with fresh inputs, and eager steps between them, give the eager step's bits."""
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    B, S, N, H, D, c_m, c_z = case
+    dev = torch.device("cuda", torch.cuda.current_device())
+    torch.manual_seed(11)
+    blk = GatedAttentionBlock(c_m, D, H, c_z=c_z, gating=True).to(dev).to(torch.bfloat16)
+    m = torch.randn(B, S, N, c_m, device=dev).to(torch.bfloat16).requires_grad_()
+    z = torch.randn(B, N, N, c_z, device=dev).to(torch.bfloat16).requires_grad_()
+    mask = (torch.rand(B, S, N, device=dev) < 0.9).float()
+    dout = torch.randn(B, S, N, c_m, device=dev).to(torch.bfloat16)
+    leaves = [m, z] + list(blk.parameters())
+
+    def step():
+        o = blk(m, z, mask)
+        return (o,) + tuple(torch.autograd.grad(o, leaves, dout))
+
+    step()                                    # first use of every kernel outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    for rep in range(3):
+        with torch.no_grad():
+            for t in (m, z, dout):
+                t.copy_(torch.randn_like(t))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = step()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.isfinite(b.float()).all()
+            assert torch.equal(a, b), (rep, i)
