@@ -73,6 +73,14 @@ def parse():
     ap.add_argument("--shape-sweep", action="store_true",
                     help="forward and backward times over row lengths, head dims, bias dtypes and both layouts, and "
                          "over the reference's own test shapes (test.py:82-100), as one JSON line")
+    ap.add_argument("--block", action="store_true",
+                    help="instead of the step benchmark: forward + backward of the gated row-attention block around "
+                         "the kernels (LayerNorm, projections, pair-bias projection, attention with the gate, output "
+                         "projection) beside the same block in plain torch operations, eager and replayed from a graph, "
+                         "as one JSON line")
+    ap.add_argument("--block-profile", action="store_true",
+                    help="--steps eager steps of the block through the kernels at C2's shape (S=512, N=256, H=8, D=32, "
+                         "c_m=256, c_z=128) and nothing else: the run to put under rocprofv3 --kernel-trace")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy three times: under rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE its counters give the scale of those counters")
@@ -231,6 +239,66 @@ def shape_sweep():
     print(json.dumps({"shape_sweep": {"unit": "us; rates in 1e12 scores/s", "rows": rows, "reference_test_shapes": ref}}))
 
 
+def block_bench(profile_steps=0):
+    """Forward + backward of `GatedAttentionBlock` (the MSA row attention of an Evoformer block, bf16, gradients of
+    m, z and every parameter) through the kernels and through plain torch operations, issued eagerly and replayed
+    from a torch.cuda.graph (a replay is one launch: the GPU's own time for the step)."""
+    import torch
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    dev = torch.device("cuda:0")
+
+    def timeit(fn, n):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n * 1e3
+
+    rows = []
+    shapes = ((1, 128, 256, 8, 32, 256, 128), (1, 512, 256, 8, 32, 256, 128), (1, 128, 384, 8, 32, 256, 128),
+              (1, 1024, 256, 8, 8, 64, 128))
+    for (B, S, N, H, D, c_m, c_z) in (shapes[1:2] if profile_steps else shapes):
+        torch.manual_seed(1)
+        blk = GatedAttentionBlock(c_m, D, H, c_z=c_z, gating=True).to(dev).to(torch.bfloat16)
+        m = torch.randn(B, S, N, c_m, device=dev).to(torch.bfloat16).requires_grad_()
+        z = torch.randn(B, N, N, c_z, device=dev).to(torch.bfloat16).requires_grad_()
+        mask = (torch.rand(B, S, N, device=dev) < 0.9).float()
+        dout = torch.randn(B, S, N, c_m, device=dev).to(torch.bfloat16)
+        leaves = [m, z] + list(blk.parameters())
+        row = {"shape": {"B": B, "S": S, "N": N, "H": H, "D": D, "c_m": c_m, "c_z": c_z}}
+        if profile_steps:
+            for _ in range(5 + profile_steps):
+                torch.autograd.grad(blk(m, z, mask), leaves, dout)
+            torch.cuda.synchronize()
+            print(json.dumps({"block_profile": {"shape": row["shape"], "steps": profile_steps, "warmup": 5}}))
+            return
+        for name, fwd in (("kernels", blk.forward), ("plain_torch", blk.forward_eager)):
+            def step():
+                return torch.autograd.grad(fwd(m, z, mask), leaves, dout)
+            t_end = time.perf_counter() + 0.5
+            while time.perf_counter() < t_end:
+                step()
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            step()
+            torch.cuda.synchronize()
+            peak = torch.cuda.max_memory_allocated() - base
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            row[name] = {"eager_us": round(timeit(step, 20), 1), "graph_replay_us": round(timeit(graph.replay, 20), 1),
+                         "peak_bytes_beyond_inputs": int(peak)}
+            del graph
+        rows.append(row)
+    print(json.dumps({"block": {"what": "GatedAttentionBlock forward + backward, bf16, one MI355X", "rows": rows}}))
+
+
 def cpu_baseline(cfg, shape, budget_s=15.0, with_bias=True):
     """The eager oracle (fp32, chunked over S) on the host cores, on a slice of S rows."""
     import torch
@@ -265,6 +333,8 @@ def main():
         return reference_sweep()
     if args.shape_sweep:
         return shape_sweep()
+    if args.block or args.block_profile:
+        return block_bench(args.steps if args.block_profile else 0)
     import torch
     from oracle import eager
     import evoformer_triton_amd.evoformer as E

@@ -29,7 +29,8 @@ EVO_PASS_FWD, EVO_PASS_BWD = 0, 1
 EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW, EVO_EHIP = 0, -1, -2, -3, -4, -5, -100
 
 EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_prep_bytes", "evoattn_bwd_workspace_bytes",
-           "evoattn_fwd", "evoattn_fwd_static", "evoattn_bwd", "evoattn_path", "evoattn_kernels")
+           "evoattn_fwd", "evoattn_fwd_static", "evoattn_bwd", "evoattn_path", "evoattn_kernels",
+           "evoattn_layernorm_fwd", "evoattn_layernorm_bwd_workspace_bytes", "evoattn_layernorm_bwd")
 EVOATTN_STATIC_PREP_BYTES = 16 << 20
 
 
@@ -92,6 +93,13 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_fwd_static.argtypes = [P, ctypes.c_void_p]
     lib.evoattn_bwd.restype = ctypes.c_int
     lib.evoattn_bwd.argtypes = [P, ctypes.c_void_p]
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+    lib.evoattn_layernorm_fwd.restype = ctypes.c_int
+    lib.evoattn_layernorm_fwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i32, i32, ctypes.c_float, vp]
+    lib.evoattn_layernorm_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.evoattn_layernorm_bwd_workspace_bytes.argtypes = [i64, i32, i32]
+    lib.evoattn_layernorm_bwd.restype = ctypes.c_int
+    lib.evoattn_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, i64, i32, i32, vp]
     lib.evoattn_path.restype = ctypes.c_char_p
     lib.evoattn_kernels.restype = ctypes.c_char_p
     lib.evoattn_path.argtypes = [P, ctypes.c_int]

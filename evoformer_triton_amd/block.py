@@ -4,7 +4,9 @@ The reference stops at the attention itself and returns O ungated (evoformer.py:
 Evoformer block the steps around it are a LayerNorm, the Q/K/V and gate projections, the
 pair-bias projection from the pair representation, sigmoid(gate) * O and the output
 projection.  This module does those with the library GEMMs (torch.nn.functional.linear is
-hipBLASLt on ROCm) and lays their results out so that the kernels read them as they fall:
+hipBLASLt on ROCm; the weight gradients are summed over slices of the rows, which as single
+GEMMs would leave most of the chip idle) and this package's LayerNorm kernels, and lays the
+results out so that the attention kernels read them as they fall:
 
   * Q, K, V and the gate come out of four Linear layers as [B,S,N,H*D], which viewed as
     [B,S,N,H,D] is the per-head ("ds4sci") layout of the kernels: no permute, no copy;
@@ -23,7 +25,136 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .evoformer import evoformer_attention
+from . import _lib
+from .evoformer import _DTYPES, _alloc_bytes, _on_device, _ptr, _stream, evoformer_attention
+
+
+def _row_slices(rows: int, n_out: int, n_in: int) -> int:
+    """Slices of the rows a weight gradient is summed over.  The gradient of an [n_out, n_in] weight is
+    one small matrix summed over all rows of the activations: as one library GEMM it has a handful of
+    output tiles (four of 128 x 128 for 256 x 256) for a chip of 256 CUs.  Summed per slice of the rows
+    as a batched GEMM and added up afterwards it fills the chip (32 768 rows, 256 x 256, bf16: 113 us as
+    one GEMM, 33 us in 8 to 128 slices; 131 072 rows: 325 against 38 us in 128)."""
+    tiles = -(-n_out // 128) * -(-n_in // 128)
+    g = 1
+    while g * tiles < 512 and rows % (2 * g) == 0 and rows // (2 * g) >= 256:
+        g *= 2
+    return g
+
+
+def _weight_grad(dy2: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
+    """dy2^T x2 ([rows, n_out], [rows, n_in] -> [n_out, n_in]) summed over slices of the rows."""
+    rows, g = dy2.shape[0], _row_slices(dy2.shape[0], dy2.shape[1], x2.shape[1])
+    if g == 1:
+        return dy2.t() @ x2
+    part = torch.bmm(dy2.view(g, rows // g, -1).transpose(1, 2), x2.view(g, rows // g, -1))
+    return part.sum(0, dtype=torch.float32).to(x2.dtype)
+
+
+class _Projections(torch.autograd.Function):
+    """Several Linear layers of one input (Q, K, V and the gate of the normalised representation):
+    forward(x, w0, b0, w1, b1, ...) -> (x w0^T + b0, x w1^T + b1, ...).  The gradient of the input
+    accumulates inside the GEMMs (`addmm_`) instead of as additions of full-size tensors after
+    them; the weight gradients are summed over slices of the rows (see _row_slices)."""
+
+    @staticmethod
+    def forward(ctx, x, *params):
+        ws, bs = params[0::2], params[1::2]
+        ctx.save_for_backward(x, *ws)
+        ctx.has_bias = tuple(b is not None for b in bs)
+        return tuple(torch.nn.functional.linear(x, w, b) for w, b in zip(ws, bs))
+
+    @staticmethod
+    def backward(ctx, *dys):
+        x, *ws = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        dx, grads = None, []
+        for i, (w, dy) in enumerate(zip(ws, dys)):
+            dy2 = dy.reshape(-1, dy.shape[-1])
+            if ctx.needs_input_grad[0]:
+                dx = dy2 @ w if dx is None else dx.addmm_(dy2, w)
+            grads.append(_weight_grad(dy2, x2) if ctx.needs_input_grad[1 + 2 * i] else None)
+            grads.append(dy2.sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[2 + 2 * i] else None)
+        return (None if dx is None else dx.view(x.shape), *grads)
+
+
+class _Linear(torch.autograd.Function):
+    """x W^T + b with the weight gradient summed over slices of the rows (see _row_slices); forward and
+    input gradient are the library's GEMMs as torch.nn.functional.linear calls them."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dy2, x2 = dy.reshape(-1, dy.shape[-1]), x.reshape(-1, x.shape[-1])
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = (dy2 @ weight).view(x.shape)
+        if ctx.needs_input_grad[1]:
+            dw = _weight_grad(dy2, x2)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = dy2.sum(0)
+        return dx, dw, db
+
+
+def _linear(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
+    return _Linear.apply(x, layer.weight, layer.bias)
+
+
+class _LayerNorm(torch.autograd.Function):
+    """LayerNorm over the last dimension through the library's kernels (evoattn_layernorm_fwd / _bwd): x and y
+    cross HBM once in the forward, x, dy and dx once in the backward; the gradients of weight and bias are summed
+    in a fixed order."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        lib = _lib.load()
+        xc = x.contiguous()
+        cols = xc.shape[-1]
+        rows = xc.numel() // cols
+        w = None if weight is None else weight.contiguous()
+        b = None if bias is None else bias.contiguous()
+        with _on_device(xc.device):
+            y = torch.empty_like(xc)
+            mean = torch.empty((rows,), device=xc.device, dtype=torch.float32)
+            rstd = torch.empty((rows,), device=xc.device, dtype=torch.float32)
+            _lib.check(lib.evoattn_layernorm_fwd(_ptr(xc), _ptr(w), _ptr(b), _ptr(y), _ptr(mean), _ptr(rstd), rows, cols,
+                                                 _DTYPES[xc.dtype], float(eps), _stream(xc.device)), "evoattn_layernorm_fwd")
+        ctx.save_for_backward(xc, w, mean, rstd)
+        ctx.has_bias = bias is not None
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        xc, w, mean, rstd = ctx.saved_tensors
+        cols = xc.shape[-1]
+        rows = xc.numel() // cols
+        dyc = dy.contiguous()
+        need_x, need_w, need_b = ctx.needs_input_grad[0], w is not None and ctx.needs_input_grad[1], ctx.has_bias and ctx.needs_input_grad[2]
+        if not (need_x or need_w or need_b):
+            return None, None, None, None
+        with _on_device(xc.device):
+            dx = torch.empty_like(xc) if need_x else None
+            dw = torch.empty((cols,), device=xc.device, dtype=xc.dtype) if need_w else None
+            db = torch.empty((cols,), device=xc.device, dtype=xc.dtype) if need_b else None
+            ws = _alloc_bytes(lib.evoattn_layernorm_bwd_workspace_bytes(rows, cols, _DTYPES[xc.dtype]), xc.device) if need_w or need_b else None
+            _lib.check(lib.evoattn_layernorm_bwd(_ptr(dyc), _ptr(xc), _ptr(w), _ptr(mean), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(db),
+                                                 _ptr(ws), 0 if ws is None else ws.numel(), rows, cols, _DTYPES[xc.dtype],
+                                                 _stream(xc.device)), "evoattn_layernorm_bwd")
+        return dx, dw, db, None
+
+
+def _layer_norm(layer: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
+    w, b = layer.weight, layer.bias
+    if w is not None and w.dtype != x.dtype:
+        return layer(x)          # mixed dtypes: the framework's
+    return _LayerNorm.apply(x, w, b, layer.eps)
 
 
 class GatedAttentionBlock(nn.Module):
@@ -53,19 +184,26 @@ class GatedAttentionBlock(nn.Module):
         else:
             self.layer_norm_z = self.linear_z = None
 
-    def operands(self, m: torch.Tensor, z: Optional[torch.Tensor], mask: Optional[torch.Tensor]):
+    def operands(self, m: torch.Tensor, z: Optional[torch.Tensor], mask: Optional[torch.Tensor], plain: bool = False):
         """Q, K, V, gate [B,S,N,H,D] (views of the projections), additive mask [B,S,1,1,N],
-        bias [B,1,H,N,N]."""
+        bias [B,1,H,N,N].  `plain`: the framework's LayerNorm and Linear throughout (what
+        `forward_eager` uses), else the library's LayerNorm kernels and the projections with
+        their weight gradients summed over slices of the rows."""
         B, S, N, _ = m.shape
         H, D = self.no_heads, self.c_hidden
-        x = self.layer_norm_m(m)
-        q = self.linear_q(x).view(B, S, N, H, D)
-        k = self.linear_k(x).view(B, S, N, H, D)
-        v = self.linear_v(x).view(B, S, N, H, D)
-        g = self.linear_g(x).view(B, S, N, H, D) if self.linear_g is not None else None
+        norm = (lambda layer, t: layer(t)) if plain or not m.is_cuda else _layer_norm
+        lin = (lambda layer, t: layer(t)) if plain else _linear
+        x = norm(self.layer_norm_m, m)
+        layers = [self.linear_q, self.linear_k, self.linear_v] + ([self.linear_g] if self.linear_g is not None else [])
+        if plain:
+            outs = [layer(x) for layer in layers]
+        else:
+            outs = _Projections.apply(x, *(t for layer in layers for t in (layer.weight, layer.bias)))
+        q, k, v = (t.view(B, S, N, H, D) for t in outs[:3])
+        g = outs[3].view(B, S, N, H, D) if self.linear_g is not None else None
         bias = None
         if z is not None and self.linear_z is not None:
-            bias = self.linear_z(self.layer_norm_z(z)).permute(0, 3, 1, 2).unsqueeze(1).contiguous().to(q.dtype)
+            bias = lin(self.linear_z, norm(self.layer_norm_z, z)).permute(0, 3, 1, 2).unsqueeze(1).contiguous().to(q.dtype)
         add_mask = None
         if mask is not None:
             add_mask = (self.inf * (mask.to(torch.float32) - 1.0)).view(B, S, 1, 1, N)
@@ -75,13 +213,13 @@ class GatedAttentionBlock(nn.Module):
         B, S, N, _ = m.shape
         q, k, v, g, add_mask, bias = self.operands(m, z, mask)
         o = evoformer_attention(q, k, v, add_mask, bias, layout="ds4sci", gate=g)
-        return self.linear_o(o.reshape(B, S, N, self.no_heads * self.c_hidden))
+        return _linear(self.linear_o, o.reshape(B, S, N, self.no_heads * self.c_hidden))
 
     def forward_eager(self, m: torch.Tensor, z: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None):
         """The same block with plain torch operations (the formula of the reference's oracle,
         test.py:47-57, with the per-head view): what `forward` is tested against."""
         B, S, N, _ = m.shape
-        q, k, v, g, add_mask, bias = self.operands(m, z, mask)
+        q, k, v, g, add_mask, bias = self.operands(m, z, mask, plain=True)
         qh, kh, vh = (t.permute(0, 1, 3, 2, 4) for t in (q, k, v))              # [B,S,H,N,D]
         s = torch.matmul(qh * self.c_hidden ** -0.5, kh.transpose(-1, -2)).float()
         if bias is not None:

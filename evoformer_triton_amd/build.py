@@ -36,7 +36,7 @@ VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans"]
 
 def _units():
     units = [("api", "api.hip", []), ("generic", "generic.hip", []), ("dispatch", "dispatch.hip", []),
-             ("prep", "prep.hip", [])]
+             ("prep", "prep.hip", []), ("layernorm", "layernorm.hip", [])]
     for d in HEAD_DIMS:
         units.append((f"mfma_fwd_d{d}", "mfma_fwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))
         units.append((f"mfma_bwd_d{d}", "mfma_bwd.hip", [f"-DEVO_D={d}", *VGPR_FORM]))

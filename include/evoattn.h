@@ -192,6 +192,25 @@ const char *evoattn_path(const EvoAttnParams *p, int pass);
  * "mfma_dq_ring,mfma_dkdv", "mfma_dq_wide,mfma_dkdv", "generic"); for reports and profiles. */
 const char *evoattn_kernels(const EvoAttnParams *p, int pass);
 
+/* ---- LayerNorm of the block around the attention -------------------------------------------
+ * No counterpart in the reference's operator, which starts at Q, K, V (evoformer.py:640-651): in
+ * an Evoformer block the representation is normalised before the Q, K, V and gate projections and
+ * the pair representation before the bias projection; these entry points do that normalisation
+ * (over the last dimension of a dense [rows, cols] array) at the rate of HBM.
+ *   dtype  EVO_BF16 / EVO_F16 / EVO_F32: x, y, gamma, beta, dy, dx, dgamma, dbeta
+ *   cols   a multiple of 16 bytes' worth of elements, at most 2048 (1024 for fp32)
+ *   gamma, beta, dx, dgamma, dbeta may be NULL (weight 1, bias 0; gradient not wanted)
+ *   mean, rstd  [rows] fp32: written by the forward, read by the backward
+ * All pointers 16-byte aligned.  The backward sums the gradients of gamma and beta through
+ * `workspace` (evoattn_layernorm_bwd_workspace_bytes) in a fixed order: bit-reproducible.
+ * Nothing is allocated or synchronised; everything runs on `hip_stream`. */
+int evoattn_layernorm_fwd(const void *x, const void *gamma, const void *beta, void *y, float *mean, float *rstd,
+                          int64_t rows, int32_t cols, int32_t dtype, float eps, void *hip_stream);
+size_t evoattn_layernorm_bwd_workspace_bytes(int64_t rows, int32_t cols, int32_t dtype);
+int evoattn_layernorm_bwd(const void *dy, const void *x, const void *gamma, const float *mean, const float *rstd,
+                          void *dx, void *dgamma, void *dbeta, void *workspace, size_t workspace_bytes,
+                          int64_t rows, int32_t cols, int32_t dtype, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -246,3 +246,23 @@ def test_header_is_plain_c_and_the_library_loads_from_c(tmp_path):
     out = subprocess.run([str(exe), _lib.LIB_PATH], capture_output=True, text=True, timeout=60)
     assert out.returncode == 0, out.stderr
     assert f"sizeof(EvoAttnParams) = {ctypes.sizeof(EvoAttnParams)}" in out.stdout
+
+
+def test_layernorm_entry_points_validate_on_the_host(lib):
+    """Argument errors of the LayerNorm entry points are found before anything is launched."""
+    import ctypes
+    buf = ctypes.create_string_buffer(4096 + 16)
+    a = (ctypes.addressof(buf) + 15) & ~15
+    fwd = lambda x=a, y=a, mean=a, rstd=a, rows=4, cols=64, dtype=_lib.EVO_BF16, eps=1e-5, gamma=None: \
+        lib.evoattn_layernorm_fwd(x, gamma, None, y, mean, rstd, rows, cols, dtype, eps, None)
+    assert fwd(x=None) == _lib.EVO_EINVAL and fwd(cols=0) == _lib.EVO_EINVAL and fwd(dtype=7) == _lib.EVO_EINVAL
+    assert fwd(cols=12) == _lib.EVO_EALIGN and fwd(x=a + 2) == _lib.EVO_EALIGN and fwd(gamma=a + 4) == _lib.EVO_EALIGN
+    assert fwd(cols=4096) == _lib.EVO_EUNSUPPORTED and fwd(cols=2048, dtype=_lib.EVO_F32) == _lib.EVO_EUNSUPPORTED
+    assert fwd(rows=0) == 0                                   # no rows: nothing to launch
+    assert lib.evoattn_layernorm_bwd_workspace_bytes(100, 256, _lib.EVO_BF16) == 1024 * 2 * 256 * 4
+    assert lib.evoattn_layernorm_bwd_workspace_bytes(100, 12, _lib.EVO_BF16) == 0
+    bwd = lambda dx=a, dgamma=None, ws=None, ws_bytes=0, cols=64: \
+        lib.evoattn_layernorm_bwd(a, a, None, a, a, dx, dgamma, None, ws, ws_bytes, 4, cols, _lib.EVO_BF16, None)
+    assert bwd(dx=None) == _lib.EVO_EINVAL                    # no output asked for
+    assert bwd(dgamma=a) == _lib.EVO_EWORKSPACE and bwd(dgamma=a, ws=a, ws_bytes=100) == _lib.EVO_EWORKSPACE
+    assert bwd(cols=20) == _lib.EVO_EALIGN

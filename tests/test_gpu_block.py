@@ -136,3 +136,49 @@ def test_block_step_under_graph_capture(case):
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.isfinite(b.float()).all()
             assert torch.equal(a, b), (rep, i)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1000, 256), (777, 128), (33, 64), (5, 8), (130, 2048), (64, 520), (3, 4, 5, 40), (70000, 64)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_layernorm_kernels_match_torch(shape, dtype):
+    """The library's LayerNorm (forward, dx, and the weight and bias gradients) against torch's in fp32 on the
+    same (rounded) inputs, to the rounding of the output dtype."""
+    from evoformer_triton_amd.block import _LayerNorm
+    if dtype == torch.float32 and shape[-1] > 1024:
+        pytest.skip("fp32 rows hold at most 1024 columns")
+    dev = torch.device("cuda", torch.cuda.current_device())
+    g = torch.Generator().manual_seed(7)
+    cols = shape[-1]
+    x = (torch.randn(shape, generator=g) * 1.5 + 0.3).to(dtype).to(dev).requires_grad_()
+    w = (1.0 + 0.2 * torch.randn(cols, generator=g)).to(dtype).to(dev).requires_grad_()
+    b = (0.1 * torch.randn(cols, generator=g)).to(dtype).to(dev).requires_grad_()
+    dy = torch.randn(shape, generator=g).to(dtype).to(dev)
+    y = _LayerNorm.apply(x, w, b, 1e-5)
+    got = (y,) + torch.autograd.grad(y, [x, w, b], dy)
+    x32, w32, b32 = (t.detach().float().requires_grad_() for t in (x, w, b))
+    y32 = torch.nn.functional.layer_norm(x32, (cols,), w32, b32, 1e-5)
+    want = (y32,) + torch.autograd.grad(y32, [x32, w32, b32], dy.float())
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
+    for name, a, c in zip(("y", "dx", "dweight", "dbias"), got, want):
+        assert a.dtype == dtype and a.shape == c.shape, name
+        err = (a.float() - c).abs().max().item()
+        assert err <= 1.5 * ulp * max(1.0, c.abs().max().item()), (name, err, c.abs().max().item())
+    # twice the same bits (the sums over rows have a fixed order)
+    y2 = _LayerNorm.apply(x, w, b, 1e-5)
+    again = (y2,) + torch.autograd.grad(y2, [x, w, b], dy)
+    for a, c in zip(got, again):
+        assert torch.equal(a, c)
+
+
+def test_layernorm_without_weight_or_input_gradient():
+    from evoformer_triton_amd.block import _LayerNorm
+    dev = torch.device("cuda", torch.cuda.current_device())
+    x = torch.randn(50, 96, device=dev).to(torch.bfloat16)
+    y = _LayerNorm.apply(x, None, None, 1e-5)
+    want = torch.nn.functional.layer_norm(x.float(), (96,))
+    assert (y.float() - want).abs().max().item() <= 2.0 ** -7 * want.abs().max().item()
+    w = torch.ones(96, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    y = _LayerNorm.apply(x, w, None, 1e-5)          # x takes no gradient: only the weight's sum is formed
+    (dw,) = torch.autograd.grad(y, [w], torch.ones_like(y))
+    assert (dw.float() - want.sum(0)).abs().max().item() <= 2.0 ** -7 * max(1.0, want.sum(0).abs().max().item())

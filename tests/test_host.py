@@ -129,3 +129,49 @@ def test_head_dim_padding_rule():
     x = torch.ones(2, 3, 24)
     y = E._padded(x, 32)
     assert y.shape == (2, 3, 32) and float(y[..., 24:].abs().sum()) == 0.0 and E._padded(x, 24) is x
+
+
+@pytest.mark.parametrize("shape,n_out,with_bias", [((2, 8, 256, 64), 32, True), ((4096, 48), 40, False), ((3, 5, 7, 16), 8, True)])
+def test_block_linear_gradients_match_torch(shape, n_out, with_bias):
+    """The block's projections sum their weight gradient over slices of the rows: same values as
+    torch.nn.functional.linear's gradients (fp32, on the CPU), for sliced and unsliced row counts."""
+    from evoformer_triton_amd import block
+    rows = 1
+    for d in shape[:-1]:
+        rows *= d
+    assert block._row_slices(4096, 32, 64) == 16 and block._row_slices(105, 8, 16) == 1
+    assert (block._row_slices(rows, n_out, shape[-1]) > 1) == (rows == 4096)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(shape, generator=g, requires_grad=True)
+    w = torch.randn((n_out, shape[-1]), generator=g, requires_grad=True)
+    b = torch.randn((n_out,), generator=g, requires_grad=True) if with_bias else None
+    dy = torch.randn(shape[:-1] + (n_out,), generator=g)
+    leaves = [x, w] + ([b] if with_bias else [])
+    y0 = torch.nn.functional.linear(x, w, b)
+    want = torch.autograd.grad(y0, leaves, dy)
+    y1 = block._Linear.apply(x, w, b)
+    got = torch.autograd.grad(y1, leaves, dy)
+    assert torch.equal(y0, y1)
+    for a, c in zip(got, want):
+        assert a.shape == c.shape
+        assert (a - c).abs().max().item() <= 1e-4 * max(1.0, c.abs().max().item())
+
+
+def test_block_projections_of_one_input_match_torch():
+    """Q, K, V and gate projections as one autograd node (the input gradient accumulated inside the GEMMs):
+    same outputs and gradients as four torch Linear layers."""
+    from evoformer_triton_amd import block
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn((2, 8, 256, 48), generator=g, requires_grad=True)
+    ws = [torch.randn((n, 48), generator=g, requires_grad=True) for n in (32, 32, 32, 40)]
+    bs = [None, None, None, torch.randn((40,), generator=g, requires_grad=True)]
+    dys = [torch.randn((2, 8, 256, w.shape[0]), generator=g) for w in ws]
+    leaves = [x] + ws + [bs[3]]
+    want_y = [torch.nn.functional.linear(x, w, b) for w, b in zip(ws, bs)]
+    want = torch.autograd.grad(want_y, leaves, dys)
+    got_y = block._Projections.apply(x, *(t for w, b in zip(ws, bs) for t in (w, b)))
+    got = torch.autograd.grad(got_y, leaves, dys)
+    for a, c in zip(got_y, want_y):
+        assert torch.equal(a, c)
+    for a, c in zip(got, want):
+        assert a.shape == c.shape and (a - c).abs().max().item() <= 1e-4 * max(1.0, c.abs().max().item())
