@@ -30,7 +30,8 @@ EVO_OK, EVO_EINVAL, EVO_EUNSUPPORTED, EVO_EALIGN, EVO_EWORKSPACE, EVO_EOVERFLOW,
 
 EXPORTS = ("evoattn_version", "evoattn_strerror", "evoattn_check", "evoattn_prep_bytes", "evoattn_bwd_workspace_bytes",
            "evoattn_fwd", "evoattn_fwd_static", "evoattn_bwd", "evoattn_path", "evoattn_kernels",
-           "evoattn_layernorm_fwd", "evoattn_layernorm_bwd_workspace_bytes", "evoattn_layernorm_bwd")
+           "evoattn_layernorm_fwd", "evoattn_layernorm_bwd_workspace_bytes", "evoattn_layernorm_bwd",
+           "evoattn_colsum_workspace_bytes", "evoattn_colsum")
 EVOATTN_STATIC_PREP_BYTES = 16 << 20
 
 
@@ -100,6 +101,10 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_layernorm_bwd_workspace_bytes.argtypes = [i64, i32, i32]
     lib.evoattn_layernorm_bwd.restype = ctypes.c_int
     lib.evoattn_layernorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, ctypes.c_size_t, i64, i32, i32, vp]
+    lib.evoattn_colsum_workspace_bytes.restype = ctypes.c_size_t
+    lib.evoattn_colsum_workspace_bytes.argtypes = [i64, i32, i32]
+    lib.evoattn_colsum.restype = ctypes.c_int
+    lib.evoattn_colsum.argtypes = [vp, vp, vp, ctypes.c_size_t, i64, i32, i32, vp]
     lib.evoattn_path.restype = ctypes.c_char_p
     lib.evoattn_kernels.restype = ctypes.c_char_p
     lib.evoattn_path.argtypes = [P, ctypes.c_int]

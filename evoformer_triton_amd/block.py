@@ -48,7 +48,24 @@ def _weight_grad(dy2: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
     if g == 1:
         return dy2.t() @ x2
     part = torch.bmm(dy2.view(g, rows // g, -1).transpose(1, 2), x2.view(g, rows // g, -1))
-    return part.sum(0, dtype=torch.float32).to(x2.dtype)
+    return part.sum(0)          # (torch adds 16-bit inputs in fp32 and rounds the sum once)
+
+
+def _bias_grad(dy2: torch.Tensor) -> torch.Tensor:
+    """Column sums of dy2 [rows, n_out]: through the library's kernel (one pass at the rate of HBM, fp32 sums in a
+    fixed order) where it takes the shape, else torch's."""
+    rows, cols = dy2.shape
+    if rows and dy2.is_cuda and dy2.dtype in _DTYPES and dy2.is_contiguous() and dy2.data_ptr() % 16 == 0:
+        lib = _lib.load()
+        nbytes = lib.evoattn_colsum_workspace_bytes(rows, cols, _DTYPES[dy2.dtype])
+        if nbytes:
+            with _on_device(dy2.device):
+                out = torch.empty((cols,), device=dy2.device, dtype=dy2.dtype)
+                ws = _alloc_bytes(nbytes, dy2.device)
+                _lib.check(lib.evoattn_colsum(_ptr(dy2), _ptr(out), _ptr(ws), ws.numel(), rows, cols, _DTYPES[dy2.dtype],
+                                              _stream(dy2.device)), "evoattn_colsum")
+            return out
+    return dy2.sum(0)
 
 
 class _Projections(torch.autograd.Function):
@@ -74,7 +91,7 @@ class _Projections(torch.autograd.Function):
             if ctx.needs_input_grad[0]:
                 dx = dy2 @ w if dx is None else dx.addmm_(dy2, w)
             grads.append(_weight_grad(dy2, x2) if ctx.needs_input_grad[1 + 2 * i] else None)
-            grads.append(dy2.sum(0) if ctx.has_bias[i] and ctx.needs_input_grad[2 + 2 * i] else None)
+            grads.append(_bias_grad(dy2) if ctx.has_bias[i] and ctx.needs_input_grad[2 + 2 * i] else None)
         return (None if dx is None else dx.view(x.shape), *grads)
 
 
@@ -98,7 +115,7 @@ class _Linear(torch.autograd.Function):
         if ctx.needs_input_grad[1]:
             dw = _weight_grad(dy2, x2)
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            db = dy2.sum(0)
+            db = _bias_grad(dy2)
         return dx, dw, db
 
 
@@ -152,8 +169,9 @@ class _LayerNorm(torch.autograd.Function):
 
 def _layer_norm(layer: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
     w, b = layer.weight, layer.bias
-    if w is not None and w.dtype != x.dtype:
-        return layer(x)          # mixed dtypes: the framework's
+    if x.numel() == 0 or x.dtype not in _DTYPES or (w is not None and w.dtype != x.dtype) \
+            or _lib.load().evoattn_layernorm_bwd_workspace_bytes(1, x.shape[-1], _DTYPES[x.dtype]) == 0:
+        return layer(x)          # no rows, mixed dtypes, or a row length the kernels do not take: the framework's
     return _LayerNorm.apply(x, w, b, layer.eps)
 
 

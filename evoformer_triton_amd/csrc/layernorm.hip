@@ -207,13 +207,53 @@ ln_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const T *__rest
     }
 }
 
-// dgamma, dbeta = the sums of the partials over the workgroups, in a fixed order.  A workgroup takes 4
+// Column sums of a dense [rows, cols] array (the bias gradient of a Linear layer): the same walk over
+// the rows as the LayerNorm backward, one partial [cols] per workgroup.
+template <typename T, int PIECES>
+__global__ void __launch_bounds__(kLnThreads)
+colsum_kernel(const T *__restrict__ a, float *__restrict__ part, int64_t rows, int cols, int lpr) {
+    constexpr int VEC = LnVec<T>::N;
+    typedef typename LnVec<T>::type vT;
+    __shared__ float red[kLnThreads * PIECES * VEC];
+    const int tid = threadIdx.x, sub = tid % lpr, grp = tid / lpr, rpb = kLnThreads / lpr;
+    const int npieces = cols / VEC;
+    float acc[PIECES][VEC];
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[i][e] = 0.0f;
+    for (int64_t row = (int64_t)blockIdx.x * rpb + grp; row < rows; row += (int64_t)gridDim.x * rpb) {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int pc = i * lpr + sub;
+            if (pc < npieces) {
+                const vT v = *reinterpret_cast<const vT *>(a + row * cols + pc * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[i][e] += (float)v[e];
+            }
+        }
+    }
+    const int pitch = lpr * PIECES * VEC;
+#pragma unroll
+    for (int i = 0; i < PIECES; ++i)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) red[grp * pitch + (i * lpr + sub) * VEC + e] = acc[i][e];
+    __syncthreads();
+    for (int c = tid; c < cols; c += kLnThreads) {
+        float s = 0.0f;
+        for (int r2 = 0; r2 < rpb; ++r2) s += red[r2 * pitch + c];
+        part[(int64_t)blockIdx.x * cols + c] = s;
+    }
+}
+
+// dgamma, dbeta = the sums of the partials over the workgroups, in a fixed order (`narr` arrays per partial:
+// two for the LayerNorm backward, one for plain column sums, whose result goes to `dgamma`).  A workgroup takes 4
 // columns and splits the partials over 64 threads per column, four rows in flight per thread (one
 // thread per column walking over a thousand partials waits for a thousand loads in turn: 64 us).
 constexpr int kLnRedCols = 4, kLnRedSlices = 64;
 template <typename T>
 __global__ void __launch_bounds__(kLnRedCols * kLnRedSlices)
-ln_reduce_kernel(const float *__restrict__ part, int nblk, int cols, T *__restrict__ dgamma, T *__restrict__ dbeta) {
+ln_reduce_kernel(const float *__restrict__ part, int nblk, int narr, int cols, T *__restrict__ dgamma, T *__restrict__ dbeta) {
     __shared__ float red[2][kLnRedCols][kLnRedSlices];
     const int cq = threadIdx.x % kLnRedCols, rs = threadIdx.x / kLnRedCols, c = blockIdx.x * kLnRedCols + cq;
     float a[4] = {0.0f, 0.0f, 0.0f, 0.0f}, b[4] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -222,15 +262,15 @@ ln_reduce_kernel(const float *__restrict__ part, int nblk, int cols, T *__restri
         for (; k + 3 * kLnRedSlices < nblk; k += 4 * kLnRedSlices) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const float *row = part + (int64_t)(k + u * kLnRedSlices) * 2 * cols;
+                const float *row = part + (int64_t)(k + u * kLnRedSlices) * narr * cols;
                 a[u] += row[c];
-                b[u] += row[cols + c];
+                if (narr == 2) b[u] += row[cols + c];
             }
         }
         for (; k < nblk; k += kLnRedSlices) {
-            const float *row = part + (int64_t)k * 2 * cols;
+            const float *row = part + (int64_t)k * narr * cols;
             a[0] += row[c];
-            b[0] += row[cols + c];
+            if (narr == 2) b[0] += row[cols + c];
         }
     }
     red[0][cq][rs] = (a[0] + a[1]) + (a[2] + a[3]);
@@ -295,10 +335,26 @@ static int ln_bwd_launch(const void *dy, const void *x, const void *gamma, const
         if (const int rc = hip_rc()) return rc;
     }
     if (sums) {   // (no rows: no partials, the sums are zero)
-        ln_reduce_kernel<T><<<(cols + kLnRedCols - 1) / kLnRedCols, kLnRedCols * kLnRedSlices, 0, st>>>(part, rows > 0 ? (int)grid : 0, cols, (T *)dgamma, (T *)dbeta);
+        ln_reduce_kernel<T><<<(cols + kLnRedCols - 1) / kLnRedCols, kLnRedCols * kLnRedSlices, 0, st>>>(part, rows > 0 ? (int)grid : 0, 2, cols, (T *)dgamma, (T *)dbeta);
         return hip_rc();
     }
     return EVO_OK;
+}
+
+template <typename T>
+static int colsum_launch(const void *a, void *out, float *part, int64_t rows, int cols, hipStream_t st) {
+    const LnShape s = ln_shape(cols, LnVec<T>::N);
+    const unsigned grid = ln_blocks(rows, s.lpr, kLnBwdBlocks);
+    auto go = [&](auto kern) { kern<<<grid, kLnThreads, 0, st>>>((const T *)a, part, rows, cols, s.lpr); };
+    if (rows > 0) {
+        if (s.pieces == 1) go(colsum_kernel<T, 1>);
+        else if (s.pieces == 2) go(colsum_kernel<T, 2>);
+        else go(colsum_kernel<T, 4>);
+        if (const int rc = hip_rc()) return rc;
+    }
+    ln_reduce_kernel<T><<<(cols + kLnRedCols - 1) / kLnRedCols, kLnRedCols * kLnRedSlices, 0, st>>>(part, rows > 0 ? (int)grid : 0, 1, cols,
+                                                                                                  (T *)out, (T *)nullptr);
+    return hip_rc();
 }
 
 }  // namespace evo
@@ -342,6 +398,28 @@ int evoattn_layernorm_bwd(const void *dy, const void *x, const void *gamma, cons
         case EVO_BF16: return ln_bwd_launch<bf16_t>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, part, rows, cols, st);
         case EVO_F16: return ln_bwd_launch<f16_t>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, part, rows, cols, st);
         default: return ln_bwd_launch<float>(dy, x, gamma, mean, rstd, dx, dgamma, dbeta, part, rows, cols, st);
+    }
+}
+
+size_t evoattn_colsum_workspace_bytes(int64_t rows, int32_t cols, int32_t dtype) {
+    using namespace evo;
+    if (ln_check(rows, cols, dtype) != EVO_OK) return 0;
+    return (size_t)kLnBwdBlocks * (size_t)cols * sizeof(float);
+}
+
+int evoattn_colsum(const void *a, void *out, void *workspace, size_t workspace_bytes, int64_t rows, int32_t cols, int32_t dtype,
+                   void *hip_stream) {
+    using namespace evo;
+    if (const int rc = ln_check(rows, cols, dtype)) return rc;
+    if (!a || !out) return EVO_EINVAL;
+    if (ln_misaligned(a) || ln_misaligned(workspace)) return EVO_EALIGN;
+    if (!workspace || workspace_bytes < evoattn_colsum_workspace_bytes(rows, cols, dtype)) return EVO_EWORKSPACE;
+    hipStream_t st = (hipStream_t)hip_stream;
+    float *part = (float *)workspace;
+    switch (dtype) {
+        case EVO_BF16: return colsum_launch<bf16_t>(a, out, part, rows, cols, st);
+        case EVO_F16: return colsum_launch<f16_t>(a, out, part, rows, cols, st);
+        default: return colsum_launch<float>(a, out, part, rows, cols, st);
     }
 }
 

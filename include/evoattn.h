@@ -211,6 +211,14 @@ int evoattn_layernorm_bwd(const void *dy, const void *x, const void *gamma, cons
                           void *dx, void *dgamma, void *dbeta, void *workspace, size_t workspace_bytes,
                           int64_t rows, int32_t cols, int32_t dtype, void *hip_stream);
 
+/* Column sums of a dense [rows, cols] array, out[c] = sum over rows of a[r][c], in the dtype of a (fp32
+ * sums in a fixed order).  No counterpart in the reference's operator: the bias gradient of the block's
+ * Linear layers (gate and output projection), one pass over the array at the rate of HBM.  Same limits
+ * on cols and alignment as the LayerNorm entry points; `workspace` of evoattn_colsum_workspace_bytes(). */
+size_t evoattn_colsum_workspace_bytes(int64_t rows, int32_t cols, int32_t dtype);
+int evoattn_colsum(const void *a, void *out, void *workspace, size_t workspace_bytes, int64_t rows, int32_t cols,
+                   int32_t dtype, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -266,3 +266,7 @@ def test_layernorm_entry_points_validate_on_the_host(lib):
     assert bwd(dx=None) == _lib.EVO_EINVAL                    # no output asked for
     assert bwd(dgamma=a) == _lib.EVO_EWORKSPACE and bwd(dgamma=a, ws=a, ws_bytes=100) == _lib.EVO_EWORKSPACE
     assert bwd(cols=20) == _lib.EVO_EALIGN
+    assert lib.evoattn_colsum_workspace_bytes(100, 256, _lib.EVO_F16) == 1024 * 256 * 4
+    assert lib.evoattn_colsum(None, a, a, 1 << 30, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EINVAL
+    assert lib.evoattn_colsum(a, a, None, 0, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EWORKSPACE
+    assert lib.evoattn_colsum(a, a, a, 1 << 30, 4, 12, _lib.EVO_BF16, None) == _lib.EVO_EALIGN

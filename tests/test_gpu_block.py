@@ -182,3 +182,25 @@ def test_layernorm_without_weight_or_input_gradient():
     y = _LayerNorm.apply(x, w, None, 1e-5)          # x takes no gradient: only the weight's sum is formed
     (dw,) = torch.autograd.grad(y, [w], torch.ones_like(y))
     assert (dw.float() - want.sum(0)).abs().max().item() <= 2.0 ** -7 * max(1.0, want.sum(0).abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "fp16", "fp32"])
+@pytest.mark.parametrize("shape", [(1000, 256), (70001, 64), (3, 8), (513, 1032), (0, 32)], ids=lambda s: "x".join(map(str, s)))
+def test_column_sums_match_torch(shape, dtype):
+    """The bias gradient of the block's Linear layers (column sums through the library) against an fp64 sum,
+    to the rounding of the output dtype; a shape the kernel does not take (cols no multiple of 16 bytes) falls
+    back to torch."""
+    from evoformer_triton_amd import block
+    if dtype == torch.float32 and shape[1] > 1024:
+        pytest.skip("fp32 rows hold at most 1024 columns")
+    dev = torch.device("cuda", torch.cuda.current_device())
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(shape, generator=g).to(dtype).to(dev)
+    got = block._bias_grad(a)
+    want = a.double().sum(0)
+    ulp = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -20}[dtype]
+    assert got.dtype == dtype and got.shape == want.shape
+    assert (got.double() - want).abs().max().item() <= 1.5 * ulp * max(1.0, want.abs().max().item()) if shape[0] else not got.any()
+    assert torch.equal(got, block._bias_grad(a))
+    odd = torch.randn((40, 10), generator=g).to(dtype).to(dev)       # 10 columns are no multiple of 16 bytes: torch's sum
+    assert torch.equal(block._bias_grad(odd), odd.sum(0))
