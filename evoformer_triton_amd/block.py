@@ -55,7 +55,7 @@ def _bias_grad(dy2: torch.Tensor) -> torch.Tensor:
     """Column sums of dy2 [rows, n_out]: through the library's kernel (one pass at the rate of HBM, fp32 sums in a
     fixed order) where it takes the shape, else torch's."""
     rows, cols = dy2.shape
-    if rows and dy2.is_cuda and dy2.dtype in _DTYPES and dy2.is_contiguous() and dy2.data_ptr() % 16 == 0:
+    if rows and not torch.compiler.is_compiling() and dy2.is_cuda and dy2.dtype in _DTYPES and dy2.is_contiguous() and dy2.data_ptr() % 16 == 0:
         lib = _lib.load()
         nbytes = lib.evoattn_colsum_workspace_bytes(rows, cols, _DTYPES[dy2.dtype])
         if nbytes:
@@ -169,9 +169,9 @@ class _LayerNorm(torch.autograd.Function):
 
 def _layer_norm(layer: nn.LayerNorm, x: torch.Tensor) -> torch.Tensor:
     w, b = layer.weight, layer.bias
-    if x.numel() == 0 or x.dtype not in _DTYPES or (w is not None and w.dtype != x.dtype) \
+    if torch.compiler.is_compiling() or x.numel() == 0 or x.dtype not in _DTYPES or (w is not None and w.dtype != x.dtype) \
             or _lib.load().evoattn_layernorm_bwd_workspace_bytes(1, x.shape[-1], _DTYPES[x.dtype]) == 0:
-        return layer(x)          # no rows, mixed dtypes, or a row length the kernels do not take: the framework's
+        return layer(x)          # under the tracer, no rows, mixed dtypes, or a row length the kernels do not take: the framework's
     return _LayerNorm.apply(x, w, b, layer.eps)
 
 
