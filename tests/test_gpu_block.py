@@ -146,7 +146,7 @@ def test_layernorm_kernels_match_torch(shape, dtype):
     same (rounded) inputs, to the rounding of the output dtype."""
     from evoformer_triton_amd.block import _LayerNorm
     if dtype == torch.float32 and shape[-1] > 1024:
-        pytest.skip("fp32 rows hold at most 1024 columns")
+        shape = shape[:-1] + (1024,)          # fp32 rows hold at most 1024 columns
     dev = torch.device("cuda", torch.cuda.current_device())
     g = torch.Generator().manual_seed(7)
     cols = shape[-1]
@@ -192,7 +192,7 @@ def test_column_sums_match_torch(shape, dtype):
     back to torch."""
     from evoformer_triton_amd import block
     if dtype == torch.float32 and shape[1] > 1024:
-        pytest.skip("fp32 rows hold at most 1024 columns")
+        shape = (shape[0], 1024)              # fp32 rows hold at most 1024 columns
     dev = torch.device("cuda", torch.cuda.current_device())
     g = torch.Generator().manual_seed(9)
     a = torch.randn(shape, generator=g).to(dtype).to(dev)
