@@ -19,6 +19,7 @@ EVO_FLAG_PREP_VALID = 2
 EVO_FLAG_ONLY_DQ = 4
 EVO_FLAG_ONLY_DKDV = 8
 EVO_FLAG_PER_PROBLEM = 16
+EVO_FLAG_GATE_DOUT_INPLACE = 0x80
 EVO_FLAG_DEBUG_OTHER_WIDTH = 0x100
 EVO_FLAG_DEBUG_NO_KV_RING = 0x200
 EVO_FLAG_DEBUG_FWD_BIAS_TILES = 0x400
@@ -104,7 +105,7 @@ def load(path: str | None = None) -> ctypes.CDLL:
     lib.evoattn_colsum_workspace_bytes.restype = ctypes.c_size_t
     lib.evoattn_colsum_workspace_bytes.argtypes = [i64, i32, i32]
     lib.evoattn_colsum.restype = ctypes.c_int
-    lib.evoattn_colsum.argtypes = [vp, vp, vp, ctypes.c_size_t, i64, i32, i32, vp]
+    lib.evoattn_colsum.argtypes = [vp, i64, vp, vp, ctypes.c_size_t, i64, i32, i32, vp]
     lib.evoattn_path.restype = ctypes.c_char_p
     lib.evoattn_kernels.restype = ctypes.c_char_p
     lib.evoattn_path.argtypes = [P, ctypes.c_int]

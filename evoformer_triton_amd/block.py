@@ -26,7 +26,7 @@ import torch
 from torch import nn
 
 from . import _lib
-from .evoformer import _DTYPES, _alloc_bytes, _on_device, _ptr, _stream, evoformer_attention
+from .evoformer import _DTYPES, _HEAD_DIMS, _SlotAttention, _alloc_bytes, _on_device, _ptr, _stream, evoformer_attention
 
 
 def _row_slices(rows: int, n_out: int, n_in: int) -> int:
@@ -52,17 +52,19 @@ def _weight_grad(dy2: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
 
 
 def _bias_grad(dy2: torch.Tensor) -> torch.Tensor:
-    """Column sums of dy2 [rows, n_out]: through the library's kernel (one pass at the rate of HBM, fp32 sums in a
+    """Column sums of dy2 [rows, n_out] (rows may lie further apart than n_out: some columns of a wider array):
+    through the library's kernel (one pass at the rate of HBM, fp32 sums in a
     fixed order) where it takes the shape, else torch's."""
     rows, cols = dy2.shape
-    if rows and not torch.compiler.is_compiling() and dy2.is_cuda and dy2.dtype in _DTYPES and dy2.is_contiguous() and dy2.data_ptr() % 16 == 0:
+    if rows and not torch.compiler.is_compiling() and dy2.is_cuda and dy2.dtype in _DTYPES and dy2.stride(1) == 1 \
+            and dy2.stride(0) >= cols and dy2.stride(0) % 8 == 0 and dy2.data_ptr() % 16 == 0:
         lib = _lib.load()
         nbytes = lib.evoattn_colsum_workspace_bytes(rows, cols, _DTYPES[dy2.dtype])
         if nbytes:
             with _on_device(dy2.device):
                 out = torch.empty((cols,), device=dy2.device, dtype=dy2.dtype)
                 ws = _alloc_bytes(nbytes, dy2.device)
-                _lib.check(lib.evoattn_colsum(_ptr(dy2), _ptr(out), _ptr(ws), ws.numel(), rows, cols, _DTYPES[dy2.dtype],
+                _lib.check(lib.evoattn_colsum(_ptr(dy2), dy2.stride(0), _ptr(out), _ptr(ws), ws.numel(), rows, cols, _DTYPES[dy2.dtype],
                                               _stream(dy2.device)), "evoattn_colsum")
             return out
     return dy2.sum(0)
@@ -100,9 +102,10 @@ class _Linear(torch.autograd.Function):
     input gradient are the library's GEMMs as torch.nn.functional.linear calls them."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias):
+    def forward(ctx, x, weight, bias, dx_place=None):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
+        ctx.dx_place = dx_place          # where the input gradient is to be written (shaped like x, rows may lie apart)
         return torch.nn.functional.linear(x, weight, bias)
 
     @staticmethod
@@ -111,16 +114,51 @@ class _Linear(torch.autograd.Function):
         dy2, x2 = dy.reshape(-1, dy.shape[-1]), x.reshape(-1, x.shape[-1])
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
-            dx = (dy2 @ weight).view(x.shape)
+            if ctx.dx_place is not None:
+                dx = ctx.dx_place
+                torch.mm(dy2, weight, out=dx.view(-1, x.shape[-1]))
+            else:
+                dx = (dy2 @ weight).view(x.shape)
         if ctx.needs_input_grad[1]:
             dw = _weight_grad(dy2, x2)
         if ctx.has_bias and ctx.needs_input_grad[2]:
             db = _bias_grad(dy2)
-        return dx, dw, db
+        return dx, dw, db, None
 
 
-def _linear(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
-    return _Linear.apply(x, layer.weight, layer.bias)
+def _linear(layer: nn.Linear, x: torch.Tensor, dx_place: Optional[torch.Tensor] = None) -> torch.Tensor:
+    return _Linear.apply(x, layer.weight, layer.bias, dx_place)
+
+
+class _StackedProjection(torch.autograd.Function):
+    """The Q, K, V (and gate) projections of one input as a single GEMM with their weights stacked:
+    forward(x, gate_bias, w0, w1, ...) -> x [w0; w1; ...]^T (+ gate_bias on the last layer's columns), shaped
+    [..., n * out].  The input is read once instead of n times, its gradient is one GEMM over the whole
+    gradient of the result (no additions of n partial gradients), and so is the weight gradient (summed over
+    slices of the rows, see _row_slices), cut into the layers' pieces afterwards."""
+
+    @staticmethod
+    def forward(ctx, x, gate_bias, *weights):
+        w = torch.cat(weights, 0)
+        bias = None
+        if gate_bias is not None:
+            bias = torch.cat([gate_bias.new_zeros(w.shape[0] - gate_bias.shape[0]), gate_bias])
+        ctx.save_for_backward(x, w)
+        ctx.sizes = [t.shape[0] for t in weights]
+        ctx.has_bias = gate_bias is not None
+        return torch.nn.functional.linear(x, w, bias)
+
+    @staticmethod
+    def backward(ctx, dp):
+        x, w = ctx.saved_tensors
+        dp2, x2 = dp.reshape(-1, dp.shape[-1]), x.reshape(-1, x.shape[-1])
+        dx = (dp2 @ w).view(x.shape) if ctx.needs_input_grad[0] else None
+        db = _bias_grad(dp2[:, dp2.shape[1] - ctx.sizes[-1]:]) if ctx.has_bias and ctx.needs_input_grad[1] else None
+        dws = [None] * len(ctx.sizes)
+        if any(ctx.needs_input_grad[2:]):
+            dws = list(_weight_grad(dp2, x2).split(ctx.sizes, 0))
+        return (dx, db, *dws)
+
 
 
 class _LayerNorm(torch.autograd.Function):
@@ -219,16 +257,36 @@ class GatedAttentionBlock(nn.Module):
             outs = _Projections.apply(x, *(t for layer in layers for t in (layer.weight, layer.bias)))
         q, k, v = (t.view(B, S, N, H, D) for t in outs[:3])
         g = outs[3].view(B, S, N, H, D) if self.linear_g is not None else None
-        bias = None
+        bias, add_mask = self._bias_and_mask(z, mask, q.dtype, (B, S, N), norm, lin)
+        return q, k, v, g, add_mask, bias
+
+    def _bias_and_mask(self, z, mask, dtype, shape, norm, lin):
+        B, S, N = shape
+        bias = add_mask = None
         if z is not None and self.linear_z is not None:
-            bias = lin(self.linear_z, norm(self.layer_norm_z, z)).permute(0, 3, 1, 2).unsqueeze(1).contiguous().to(q.dtype)
-        add_mask = None
+            bias = lin(self.linear_z, norm(self.layer_norm_z, z)).permute(0, 3, 1, 2).unsqueeze(1).contiguous().to(dtype)
         if mask is not None:
             add_mask = (self.inf * (mask.to(torch.float32) - 1.0)).view(B, S, 1, 1, N)
-        return q, k, v, g, add_mask, bias
+        return bias, add_mask
+
+    def _slots_ok(self, m: torch.Tensor) -> bool:
+        """Whether Q, K, V and the gate can come from one GEMM and reach the kernels as slots of its result."""
+        layers = [self.linear_q, self.linear_k, self.linear_v, self.linear_o] + ([self.linear_g] if self.linear_g is not None else [])
+        return (m.is_cuda and m.numel() > 0 and not torch.compiler.is_compiling() and m.dtype in (torch.bfloat16, torch.float16)
+                and self.c_hidden in _HEAD_DIMS and all(l.weight.dtype == m.dtype for l in layers)
+                and all(l.bias is None for l in layers[:3]))
 
     def forward(self, m: torch.Tensor, z: Optional[torch.Tensor] = None, mask: Optional[torch.Tensor] = None):
         B, S, N, _ = m.shape
+        if self._slots_ok(m):
+            H, D = self.no_heads, self.c_hidden
+            gated = self.linear_g is not None
+            x = _layer_norm(self.layer_norm_m, m)
+            weights = [self.linear_q.weight, self.linear_k.weight, self.linear_v.weight] + ([self.linear_g.weight] if gated else [])
+            P = _StackedProjection.apply(x, self.linear_g.bias if gated else None, *weights).view(B, S, N, len(weights), H, D)
+            bias, add_mask = self._bias_and_mask(z, mask, m.dtype, (B, S, N), _layer_norm, _linear)
+            o, grad_slot = _SlotAttention.apply(P, add_mask, bias, gated)
+            return _linear(self.linear_o, o.reshape(B, S, N, H * D), grad_slot.view(B, S, N, H * D))
         q, k, v, g, add_mask, bias = self.operands(m, z, mask)
         o = evoformer_attention(q, k, v, add_mask, bias, layout="ds4sci", gate=g)
         return _linear(self.linear_o, o.reshape(B, S, N, self.no_heads * self.c_hidden))

@@ -17,6 +17,16 @@ static inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a
 static inline bool aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
 static inline int elem_size(int dtype) { return dtype == EVO_F32 ? 4 : 2; }
 
+
+// Elements from the first to one past the last element of a q-family tensor (= B*H*S*N*D when it is dense).
+static int64_t q_span(const EvoAttnParams &p) {
+    const int64_t st4[4] = {p.stride_b, p.stride_h, p.stride_s, p.stride_n};
+    const int64_t ext[4] = {p.B, p.H, p.S, p.N};
+    int64_t span = p.D;
+    for (int i = 0; i < 4; ++i) span += (ext[i] - 1) * st4[i];
+    return span;
+}
+
 static int check_common(const EvoAttnParams *p) {
     if (!p) return EVO_EINVAL;
     if (p->B <= 0 || p->S <= 0 || p->N <= 0 || p->H <= 0 || p->D <= 0) return EVO_EINVAL;
@@ -28,14 +38,14 @@ static int check_common(const EvoAttnParams *p) {
     if (!p->q || !p->k || !p->v || !p->o || !p->lse) return EVO_EINVAL;
     if (!(p->scale == p->scale) || p->scale <= 0.0f) return EVO_EINVAL;
     if (p->flags & ~EVO_FLAG_ALL) return EVO_EINVAL;
+    // (a second call on the same dout would apply the gate to it a second time)
+    if ((p->flags & EVO_FLAG_GATE_DOUT_INPLACE) && (p->flags & (EVO_FLAG_ONLY_DQ | EVO_FLAG_ONLY_DKDV))) return EVO_EINVAL;
     if (p->gate) {
-        // the gate is read and its products written element for element like q: that needs a dense q-family
+        // The gate is read and its products written element for element like q; the backward keeps the gradient
+        // of the ungated output in the workspace, laid out like q, gaps included: the q-family may be dense or a
+        // slot of a buffer of up to 8 such tensors (Q, K, V and the gate as one projection's result), not sparser.
         if (p->D % 8) return EVO_EUNSUPPORTED;
-        const int64_t st4[4] = {p->stride_b, p->stride_h, p->stride_s, p->stride_n};
-        const int64_t ext[4] = {p->B, p->H, p->S, p->N};
-        int64_t span = p->D;
-        for (int i = 0; i < 4; ++i) span += (ext[i] - 1) * st4[i];
-        if (span != (int64_t)p->B * p->H * p->S * p->N * p->D) return EVO_EUNSUPPORTED;
+        if (q_span(*p) > 8 * (int64_t)p->B * p->H * p->S * p->N * p->D) return EVO_EUNSUPPORTED;
     } else if (p->o_gated || p->dgate) {
         return EVO_EINVAL;
     }
@@ -277,7 +287,7 @@ static WsLayout ws_layout(const EvoAttnParams &p) {
     w.dbias_part = off;
     if (p.dbias && !dq_writes_dbias(p)) off += align_up((size_t)w.n_chunks * p.B * p.H * p.N * p.N * 4);
     w.dout_ungated = off;
-    if (p.gate) off += align_up(rows * p.D * (size_t)elem_size(p.dtype));
+    if (p.gate && !(p.flags & EVO_FLAG_GATE_DOUT_INPLACE)) off += align_up((size_t)q_span(p) * (size_t)elem_size(p.dtype));
     w.total = off;
     return w;
 }
@@ -453,8 +463,10 @@ int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
     // backward below runs on the former.
     EvoAttnParams ungated = *p0;
     if (p0->gate) {
-        if ((rc = launch_gate_bwd(*p0, ws + w.dout_ungated, st))) return rc;
-        ungated.dout = ws + w.dout_ungated;
+        // (in place: a thread reads its 8 elements of dout before it writes them)
+        void *d_o = (p0->flags & EVO_FLAG_GATE_DOUT_INPLACE) ? const_cast<void *>(p0->dout) : (void *)(ws + w.dout_ungated);
+        if ((rc = launch_gate_bwd(*p0, d_o, st))) return rc;
+        ungated.dout = d_o;
         ungated.gate = nullptr;
     }
     const EvoAttnParams *p = &ungated;

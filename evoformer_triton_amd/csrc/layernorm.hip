@@ -211,7 +211,7 @@ ln_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x, const T *__rest
 // the rows as the LayerNorm backward, one partial [cols] per workgroup.
 template <typename T, int PIECES>
 __global__ void __launch_bounds__(kLnThreads)
-colsum_kernel(const T *__restrict__ a, float *__restrict__ part, int64_t rows, int cols, int lpr) {
+colsum_kernel(const T *__restrict__ a, float *__restrict__ part, int64_t rows, int cols, int64_t row_stride, int lpr) {
     constexpr int VEC = LnVec<T>::N;
     typedef typename LnVec<T>::type vT;
     __shared__ float red[kLnThreads * PIECES * VEC];
@@ -227,7 +227,7 @@ colsum_kernel(const T *__restrict__ a, float *__restrict__ part, int64_t rows, i
         for (int i = 0; i < PIECES; ++i) {
             const int pc = i * lpr + sub;
             if (pc < npieces) {
-                const vT v = *reinterpret_cast<const vT *>(a + row * cols + pc * VEC);
+                const vT v = *reinterpret_cast<const vT *>(a + row * row_stride + pc * VEC);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) acc[i][e] += (float)v[e];
             }
@@ -342,10 +342,10 @@ static int ln_bwd_launch(const void *dy, const void *x, const void *gamma, const
 }
 
 template <typename T>
-static int colsum_launch(const void *a, void *out, float *part, int64_t rows, int cols, hipStream_t st) {
+static int colsum_launch(const void *a, void *out, float *part, int64_t rows, int cols, int64_t row_stride, hipStream_t st) {
     const LnShape s = ln_shape(cols, LnVec<T>::N);
     const unsigned grid = ln_blocks(rows, s.lpr, kLnBwdBlocks);
-    auto go = [&](auto kern) { kern<<<grid, kLnThreads, 0, st>>>((const T *)a, part, rows, cols, s.lpr); };
+    auto go = [&](auto kern) { kern<<<grid, kLnThreads, 0, st>>>((const T *)a, part, rows, cols, row_stride, s.lpr); };
     if (rows > 0) {
         if (s.pieces == 1) go(colsum_kernel<T, 1>);
         else if (s.pieces == 2) go(colsum_kernel<T, 2>);
@@ -407,19 +407,20 @@ size_t evoattn_colsum_workspace_bytes(int64_t rows, int32_t cols, int32_t dtype)
     return (size_t)kLnBwdBlocks * (size_t)cols * sizeof(float);
 }
 
-int evoattn_colsum(const void *a, void *out, void *workspace, size_t workspace_bytes, int64_t rows, int32_t cols, int32_t dtype,
-                   void *hip_stream) {
+int evoattn_colsum(const void *a, int64_t row_stride, void *out, void *workspace, size_t workspace_bytes, int64_t rows, int32_t cols,
+                   int32_t dtype, void *hip_stream) {
     using namespace evo;
     if (const int rc = ln_check(rows, cols, dtype)) return rc;
-    if (!a || !out) return EVO_EINVAL;
+    if (!a || !out || row_stride < cols) return EVO_EINVAL;
+    if (row_stride % (16 / ln_elem_bytes(dtype))) return EVO_EALIGN;
     if (ln_misaligned(a) || ln_misaligned(workspace)) return EVO_EALIGN;
     if (!workspace || workspace_bytes < evoattn_colsum_workspace_bytes(rows, cols, dtype)) return EVO_EWORKSPACE;
     hipStream_t st = (hipStream_t)hip_stream;
     float *part = (float *)workspace;
     switch (dtype) {
-        case EVO_BF16: return colsum_launch<bf16_t>(a, out, part, rows, cols, st);
-        case EVO_F16: return colsum_launch<f16_t>(a, out, part, rows, cols, st);
-        default: return colsum_launch<float>(a, out, part, rows, cols, st);
+        case EVO_BF16: return colsum_launch<bf16_t>(a, out, part, rows, cols, row_stride, st);
+        case EVO_F16: return colsum_launch<f16_t>(a, out, part, rows, cols, row_stride, st);
+        default: return colsum_launch<float>(a, out, part, rows, cols, row_stride, st);
     }
 }
 

@@ -291,19 +291,9 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
     if Dp != D:
         dQ, dK, dV = (t[..., :D].contiguous() for t in (dQ, dK, dV))
     if dbias is not None:
-        shape, dtype = bias_orig
-        dbias = dbias.reshape(B, 1, H, N, N)                    # :860
-        if shape[0] == 1 and B > 1:
-            dbias = dbias.sum(0, keepdim=True)
-        dbias = dbias.to(dtype)
+        dbias = _finish_dbias(dbias, bias_orig, B, H, N)
     if dmask is not None:
-        shape, dtype = mask_orig
-        dmask = dmask.reshape(B, S, 1, 1, N)
-        if shape[0] == 1 and B > 1:
-            dmask = dmask.sum(0, keepdim=True)
-        if shape[1] == 1 and S > 1:
-            dmask = dmask.sum(1, keepdim=True)
-        dmask = dmask.to(dtype)
+        dmask = _finish_dmask(dmask, mask_orig, B, S, N)
     if gate is not None:
         return dQ, dK, dV, dmask, dbias, (dgate[..., :D].contiguous() if Dp != D else dgate)
     return dQ, dK, dV, dmask, dbias
@@ -548,6 +538,117 @@ class _GatedAttention(torch.autograd.Function):
         dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Q, K, V, mask, bias, O, lse, prep, ctx.layout, ctx.mask_meta,
                                                     ctx.bias_meta, ctx.needs_input_grad[3], ctx.needs_input_grad[4], gate=gate)
         return dQ, dK, dV, dmask, dbias, dgate, None
+
+
+def _finish_dbias(dbias, bias_orig, B, H, N):
+    shape, dtype = bias_orig
+    dbias = dbias.reshape(B, 1, H, N, N)                        # evoformer.py:860
+    if shape[0] == 1 and B > 1:
+        dbias = dbias.sum(0, keepdim=True)
+    return dbias.to(dtype)
+
+
+def _finish_dmask(dmask, mask_orig, B, S, N):
+    shape, dtype = mask_orig
+    dmask = dmask.reshape(B, S, 1, 1, N)
+    if shape[0] == 1 and B > 1:
+        dmask = dmask.sum(0, keepdim=True)
+    if shape[1] == 1 and S > 1:
+        dmask = dmask.sum(1, keepdim=True)
+    return dmask.to(dtype)
+
+
+class _SlotAttention(torch.autograd.Function):
+    """Per-head attention on Q, K, V (and the gate's logits) that are the slots 0, 1, 2 (and 3) of one
+    contiguous tensor P [B,S,N,W,H,D]: the result of one projection GEMM with the weights of the three or
+    four Linear layers stacked, which reads the block's input once instead of W times.  The kernels take the
+    slots by their strides (a token's row lies W*H*D elements from the next); nothing is copied.  Every
+    tensor the kernels lay out like Q is a slot of a buffer of that shape:
+
+        outputs OB   slot 0  O (ungated, kept for the backward)     gradients DP   slot 0  dQ
+                     slot 1  sigmoid(g) * O (returned when gated)                  slot 1  dK
+                     slot 2  the gradient coming back (dO)                         slot 2  dV
+                     slot 3  -                                                     slot 3  dgate
+
+    forward(P, res_mask, pair_bias, gated) -> (out, grad_slot): `out` is slot 1 (gated) or slot 0 as a
+    [B,S,N,H,D] view, `grad_slot` is slot 2 as such a view, for the consumer to write the gradient of `out`
+    into (a gradient that arrives elsewhere is copied there).  backward returns DP, the gradient of P, whole:
+    the projection's input and weight gradients are single GEMMs over it."""
+
+    @staticmethod
+    def forward(ctx, P, res_mask, pair_bias, gated):
+        lib = _lib.load()
+        B, S, N, W, H, D = P.shape
+        if not P.is_contiguous() or W < (4 if gated else 3) or P.dtype not in (torch.bfloat16, torch.float16) or D not in _HEAD_DIMS:
+            raise ValueError("P must be a contiguous 16-bit [B,S,N,W,H,D] tensor with W >= 3 (4 with a gate) and a head dim the library is built for")
+        mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, P.device)
+        bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, P.dtype, P.device)
+        with _on_device(P.device):
+            OB = torch.empty_like(P)
+            lse = torch.empty((B, H, S, N), device=P.device, dtype=torch.float32)
+            p = _SlotAttention._params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
+            prep = _alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), P.device)
+            p.prep, p.prep_bytes = _ptr(prep), prep.numel()
+            if gated:
+                p.gate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(OB[:, :, :, 1])
+            _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(P.device)), "evoattn_fwd")
+        ctx.save_for_backward(P, mask, bias, lse, prep)
+        # Not among the saved tensors, and under a version counter of its own (`.data`): the consumer writes the
+        # incoming gradient into slot 2 in place, which must not look like a change of `out` (the same memory
+        # object) to whoever saved `out` for its backward.
+        raw = OB.data
+        ctx.OB = raw
+        ctx.gated = bool(gated)
+        ctx.mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
+        ctx.bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
+        out, grad_slot = OB[:, :, :, 1 if gated else 0], raw[:, :, :, 2]
+        ctx.mark_non_differentiable(grad_slot)
+        return out, grad_slot
+
+    @staticmethod
+    def _params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse):
+        B, S, N, W, H, D = P.shape
+        p = _params(P[:, :, :, 0], P[:, :, :, 1], P[:, :, :, 2], mask, mask_kind, mstr, bias, bias_dt, bstr, OB[:, :, :, 0], lse, "ds4sci")
+        p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * W * H * D, D, N * W * H * D, W * H * D
+        return p
+
+    @staticmethod
+    def backward(ctx, dout, _unused):
+        lib = _lib.load()
+        P, mask, bias, lse, prep = ctx.saved_tensors
+        OB = ctx.OB
+        B, S, N, W, H, D = P.shape
+        mask_kind, mstr, mask_orig = ctx.mask_meta
+        bias_dt, bstr, bias_orig = ctx.bias_meta
+        slot = OB[:, :, :, 2]
+        if dout.data_ptr() != slot.data_ptr() or dout.stride() != slot.stride() or dout.dtype != P.dtype:
+            slot.copy_(dout)
+        want_dmask = bool(ctx.needs_input_grad[1] and mask is not None and mask.is_floating_point())
+        want_dbias = bool(ctx.needs_input_grad[2] and bias is not None)
+        with _on_device(P.device):
+            DP = torch.empty_like(P) if W == (4 if ctx.gated else 3) else torch.zeros_like(P)
+            p = _SlotAttention._params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
+            p.dout, p.dq, p.dk, p.dv = _ptr(slot), _ptr(DP[:, :, :, 0]), _ptr(DP[:, :, :, 1]), _ptr(DP[:, :, :, 2])
+            if ctx.gated:     # slot 2 is this Function's own memory: the gradient of the ungated output takes its place
+                p.gate, p.dgate = _ptr(P[:, :, :, 3]), _ptr(DP[:, :, :, 3])
+                p.flags |= _lib.EVO_FLAG_GATE_DOUT_INPLACE
+            dbias = dmask = None
+            if want_dbias:
+                dbias = torch.empty((B, H, N, N), device=P.device, dtype=bias.dtype)
+                p.dbias, p.dbias_dtype = _ptr(dbias), _DTYPES[bias.dtype]
+            if want_dmask:
+                dmask = torch.empty((B, S, N), device=P.device, dtype=torch.float32)
+                p.dmask = _ptr(dmask)
+            ws = _alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), P.device)
+            p.workspace, p.workspace_bytes = _ptr(ws), ws.numel()
+            p.prep, p.prep_bytes = _ptr(prep), prep.numel()
+            p.flags |= _lib.EVO_FLAG_PREP_VALID
+            _lib.check(lib.evoattn_bwd(ctypes.byref(p), _stream(P.device)), "evoattn_bwd")
+        if dbias is not None:
+            dbias = _finish_dbias(dbias, bias_orig, B, H, N)
+        if dmask is not None:
+            dmask = _finish_dmask(dmask, mask_orig, B, S, N)
+        return DP, dmask, dbias, None
 
 
 def evoformer_attention(Q, K, V, res_mask=None, pair_bias=None, layout: str = "reference", gate=None):

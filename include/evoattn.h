@@ -63,6 +63,10 @@ enum {
     /* Measurement aid: run the one-workgroup-per-(b,h,s) forms of the forward and dQ kernels
      * also where the forms that walk over a chunk of S rows apply (same results). */
     EVO_FLAG_PER_PROBLEM   = 16,
+    /* evoattn_bwd with a gate: the gradient of the ungated output, dout * sigmoid(g), overwrites `dout`
+     * instead of going to the workspace, which then does not grow by q's extent.  For a caller that owns
+     * the memory of `dout` and does not need it afterwards; not together with EVO_FLAG_ONLY_DQ / _ONLY_DKDV. */
+    EVO_FLAG_GATE_DOUT_INPLACE = 0x80,
     /* Debug switches for A/B comparisons of kernel forms (same results, other kernels); a
      * production caller leaves them clear.  All other bits of `flags` must be zero. */
     EVO_FLAG_DEBUG_OTHER_WIDTH  = 0x100,  /* one-workgroup-per-problem kernels: the other of their two workgroup widths (4 / 8 waves) */
@@ -72,7 +76,7 @@ enum {
     EVO_FLAG_DEBUG_NO_DQ_WIDE   = 0x1000, /* dQ: the kernels that split a row's keys over the waves, also without a dBias sum */
     EVO_FLAG_DEBUG_NO_DQ_SPLIT  = 0x2000  /* dQ + dBias in one kernel, also where dQ and the dBias partials come from two */
 };
-#define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x100 | 0x200 | 0x400 | 0x800 | 0x1000 | 0x2000)
+#define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x80 | 0x100 | 0x200 | 0x400 | 0x800 | 0x1000 | 0x2000)
 
 /* A problem (b, s) whose every key carries a mask value below this is a "dead row"; see lse below. */
 #define EVOATTN_SHIFT_THRESHOLD (-1.0e5f)
@@ -142,9 +146,10 @@ typedef struct EvoAttnParams {
      * ungated O in `o`, which stays the tensor the backward takes delta = <dO, O> from.
      * evoattn_bwd takes in `dout` the gradient of o_gated, forms dO = dout * sigmoid(g) and
      * dgate = dout * O * sigmoid(g) * (1 - sigmoid(g)) in one pass over the rows (dgate laid out
-     * like q; dO goes to the workspace, which grows by one tensor of q's size) and runs the
-     * attention backward on that dO.  The q-family must be dense (its four strides a permutation
-     * of a contiguous [B][S][N][H][D] or [B][H][S][N][D] tensor).  The reference returns O
+     * like q; dO goes to the workspace, laid out like q, which grows by q's extent in memory) and
+     * runs the attention backward on that dO.  The q-family may be dense or a slot of a buffer of
+     * up to 8 such tensors (Q, K, V and the gate as slices of one projection's result: strides of
+     * [B][S][N][W][H][D]), not sparser.  The reference returns O
      * ungated (evoformer.py:735); its callers apply the gate as a separate step. */
     const void *gate;
     void       *o_gated;
@@ -211,13 +216,14 @@ int evoattn_layernorm_bwd(const void *dy, const void *x, const void *gamma, cons
                           void *dx, void *dgamma, void *dbeta, void *workspace, size_t workspace_bytes,
                           int64_t rows, int32_t cols, int32_t dtype, void *hip_stream);
 
-/* Column sums of a dense [rows, cols] array, out[c] = sum over rows of a[r][c], in the dtype of a (fp32
- * sums in a fixed order).  No counterpart in the reference's operator: the bias gradient of the block's
+/* Column sums of a [rows, cols] array whose rows lie `row_stride` elements apart (cols for a dense array;
+ * more for some columns of a wider one), out[c] = sum over rows of a[r][c], in the dtype of a (fp32 sums
+ * in a fixed order).  No counterpart in the reference's operator: the bias gradient of the block's
  * Linear layers (gate and output projection), one pass over the array at the rate of HBM.  Same limits
  * on cols and alignment as the LayerNorm entry points; `workspace` of evoattn_colsum_workspace_bytes(). */
 size_t evoattn_colsum_workspace_bytes(int64_t rows, int32_t cols, int32_t dtype);
-int evoattn_colsum(const void *a, void *out, void *workspace, size_t workspace_bytes, int64_t rows, int32_t cols,
-                   int32_t dtype, void *hip_stream);
+int evoattn_colsum(const void *a, int64_t row_stride, void *out, void *workspace, size_t workspace_bytes, int64_t rows,
+                   int32_t cols, int32_t dtype, void *hip_stream);
 
 #ifdef __cplusplus
 }

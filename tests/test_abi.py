@@ -173,7 +173,11 @@ def test_every_flag_bit_is_declared_in_the_header(lib):
         p.flags = bit
         assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EINVAL
     p = good()
-    p.flags = all_bits
+    p.flags = all_bits & ~_lib.EVO_FLAG_GATE_DOUT_INPLACE
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    p.flags = _lib.EVO_FLAG_GATE_DOUT_INPLACE | _lib.EVO_FLAG_ONLY_DQ      # the gate would be applied twice
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EINVAL
+    p.flags = _lib.EVO_FLAG_GATE_DOUT_INPLACE
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
 
 
@@ -214,10 +218,17 @@ def test_gate_validation_on_the_host(lib):
     q = good()
     need_plain = lib.evoattn_bwd_workspace_bytes(ctypes.byref(q))
     assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) >= need_plain + 1 * 4 * 64 * 2 * 32 * 2   # + dO, bf16
+    p.flags = _lib.EVO_FLAG_GATE_DOUT_INPLACE                                               # dO in the place of dout
+    assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) == need_plain
+    p.flags = 0
     p.gate = 0x10008
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EALIGN
     p.gate = fake
-    p.stride_s *= 2                                                                         # rows with gaps: not dense
+    dense_ws = lib.evoattn_bwd_workspace_bytes(ctypes.byref(p))
+    p.stride_s *= 2                                              # rows with gaps (a slot of a wider buffer): the workspace's dO has them too
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) == dense_ws + 3 * 64 * 32 * 2              # three more gaps of a row's size
+    p.stride_s *= 16                                             # sparser than a slot of 8
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EUNSUPPORTED
     # the per-head layout of the same dense tensor is fine
     p = good()
@@ -267,6 +278,8 @@ def test_layernorm_entry_points_validate_on_the_host(lib):
     assert bwd(dgamma=a) == _lib.EVO_EWORKSPACE and bwd(dgamma=a, ws=a, ws_bytes=100) == _lib.EVO_EWORKSPACE
     assert bwd(cols=20) == _lib.EVO_EALIGN
     assert lib.evoattn_colsum_workspace_bytes(100, 256, _lib.EVO_F16) == 1024 * 256 * 4
-    assert lib.evoattn_colsum(None, a, a, 1 << 30, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EINVAL
-    assert lib.evoattn_colsum(a, a, None, 0, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EWORKSPACE
-    assert lib.evoattn_colsum(a, a, a, 1 << 30, 4, 12, _lib.EVO_BF16, None) == _lib.EVO_EALIGN
+    assert lib.evoattn_colsum(None, 64, a, a, 1 << 30, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EINVAL
+    assert lib.evoattn_colsum(a, 64, a, None, 0, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EWORKSPACE
+    assert lib.evoattn_colsum(a, 12, a, a, 1 << 30, 4, 12, _lib.EVO_BF16, None) == _lib.EVO_EALIGN
+    assert lib.evoattn_colsum(a, 32, a, a, 1 << 30, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EINVAL       # rows overlap
+    assert lib.evoattn_colsum(a, 68, a, a, 1 << 30, 4, 64, _lib.EVO_BF16, None) == _lib.EVO_EALIGN

@@ -202,6 +202,10 @@ def test_column_sums_match_torch(shape, dtype):
     assert got.dtype == dtype and got.shape == want.shape
     assert (got.double() - want).abs().max().item() <= 1.5 * ulp * max(1.0, want.abs().max().item()) if shape[0] else not got.any()
     assert torch.equal(got, block._bias_grad(a))
+    if shape[0]:                                                     # some columns of a wider array
+        wide = torch.randn((shape[0], 3 * shape[1]), generator=g).to(dtype).to(dev)
+        part = wide[:, shape[1]:2 * shape[1]]
+        assert torch.equal(block._bias_grad(part), block._bias_grad(part.contiguous()))
     odd = torch.randn((40, 10), generator=g).to(dtype).to(dev)       # 10 columns are no multiple of 16 bytes: torch's sum
     assert torch.equal(block._bias_grad(odd), odd.sum(0))
 
@@ -235,3 +239,58 @@ def test_block_compiles_as_one_graph():
             rel = ((a.float() - w.float()).norm() / w.float().norm().clamp_min(1e-12)).item()
             err = (a.float() - w.float()).abs().max().item()
             assert rel <= 2e-2 or err <= 2e-4, (rel, err)
+
+
+@pytest.mark.parametrize("case", [(1, 12, 256, 4, 32, True), (2, 5, 100, 2, 16, True), (1, 6, 384, 4, 32, False),
+                                  (1, 9, 128, 8, 8, True), (1, 3, 512, 2, 64, True), (1, 2, 1100, 2, 32, False)],
+                         ids=lambda c: "-".join(map(str, c)))
+def test_slot_attention_matches_the_dense_per_head_call(case):
+    """Q, K, V and the gate as slots of one [B,S,N,W,H,D] tensor (what one stacked projection GEMM produces),
+    outputs and gradients in slots of buffers of that shape: bit for bit what the per-head call gives on dense
+    copies of the slots, with the gradient arriving elsewhere (copied into its slot) and written into the slot."""
+    import evoformer_triton_amd.evoformer as E
+    B, S, N, H, D, gated = case
+    W = 4 if gated else 3
+    dev = torch.device("cuda", torch.cuda.current_device())
+    g = torch.Generator().manual_seed(13)
+    P = torch.randn((B, S, N, W, H, D), generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    bias = (torch.randn((1, 1, H, N, N), generator=g) * 0.5).to(torch.bfloat16).to(dev).requires_grad_()
+    mask = torch.where(torch.rand((B, S, 1, 1, N), generator=g) < 0.9, 0.0, -1e9).to(dev)
+    dO = torch.randn((B, S, N, H, D), generator=g).to(torch.bfloat16).to(dev)
+
+    parts = [P.detach()[:, :, :, i].contiguous().requires_grad_() for i in range(W)]
+    b2 = bias.detach().clone().requires_grad_()
+    ref = E.evoformer_attention(parts[0], parts[1], parts[2], mask, b2, layout="ds4sci", gate=parts[3] if gated else None)
+    ref_grads = torch.autograd.grad(ref, parts + [b2], dO)
+
+    out, slot = E._SlotAttention.apply(P, mask, bias, gated)
+    assert out.shape == (B, S, N, H, D) and slot.shape == out.shape and not slot.requires_grad
+    assert torch.equal(out, ref)
+    dP, db = torch.autograd.grad(out, [P, bias], dO, retain_graph=True)          # the gradient arrives elsewhere
+    for i in range(W):
+        assert torch.equal(dP[:, :, :, i], ref_grads[i]), i
+    assert torch.equal(db, ref_grads[W])
+    slot.copy_(dO)                                                               # the consumer wrote it into the slot
+    dP2, db2 = torch.autograd.grad(out, [P, bias], slot)
+    assert torch.equal(dP2, dP) and torch.equal(db2, db)
+
+
+def test_block_takes_the_slot_path_on_the_gpu():
+    """In 16-bit on the GPU the block's Q, K, V and gate come from one GEMM and reach the kernels as slots;
+    the layer-by-layer path (fp32, under the tracer) gives the same to the rounding of the dtype."""
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    dev = torch.device("cuda", torch.cuda.current_device())
+    torch.manual_seed(3)
+    blk = GatedAttentionBlock(64, 32, 4, c_z=32).to(dev).to(torch.bfloat16)
+    m = torch.randn(1, 6, 128, 64, device=dev).to(torch.bfloat16).requires_grad_()
+    z = torch.randn(1, 128, 128, 32, device=dev).to(torch.bfloat16).requires_grad_()
+    assert blk._slots_ok(m) and not blk.float()._slots_ok(m.float())
+    blk = blk.to(torch.bfloat16)
+    leaves = [m, z] + list(blk.parameters())
+    dout = torch.randn(1, 6, 128, 64, device=dev).to(torch.bfloat16)
+    new = torch.autograd.grad(blk(m, z), leaves, dout)
+    blk._slots_ok = lambda m: False
+    old = torch.autograd.grad(blk(m, z), leaves, dout)
+    for a, b in zip(new, old):
+        rel = ((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-12)).item()
+        assert rel <= 2e-2 or (a.float() - b.float()).abs().max().item() <= 2e-4, rel
