@@ -106,7 +106,10 @@ class _Linear(torch.autograd.Function):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
         ctx.dx_place = dx_place          # where the input gradient is to be written (shaped like x, rows may lie apart)
-        return torch.nn.functional.linear(x, weight, bias)
+        # (as a matrix: for an input of more dimensions whose rows lie apart torch multiplies and then adds the
+        # bias in a pass of its own)
+        y = torch.nn.functional.linear(x.reshape(-1, x.shape[-1]), weight, bias)
+        return y.view(*x.shape[:-1], weight.shape[0])
 
     @staticmethod
     def backward(ctx, dy):

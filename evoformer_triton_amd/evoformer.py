@@ -621,7 +621,9 @@ class _SlotAttention(torch.autograd.Function):
         mask_kind, mstr, mask_orig = ctx.mask_meta
         bias_dt, bstr, bias_orig = ctx.bias_meta
         slot = OB[:, :, :, 2]
-        if dout.data_ptr() != slot.data_ptr() or dout.stride() != slot.stride() or dout.dtype != P.dtype:
+        in_place = dout.data_ptr() == slot.data_ptr() and dout.dtype == slot.dtype and dout.shape == slot.shape and all(
+            n == 1 or a == b for n, a, b in zip(slot.shape, dout.stride(), slot.stride()))
+        if not in_place:
             slot.copy_(dout)
         want_dmask = bool(ctx.needs_input_grad[1] and mask is not None and mask.is_floating_point())
         want_dbias = bool(ctx.needs_input_grad[2] and bias is not None)
