@@ -244,7 +244,8 @@ def test_block_compiles_as_one_graph():
 @pytest.mark.parametrize("case", [(1, 12, 256, 4, 32, True), (2, 5, 100, 2, 16, True), (1, 6, 384, 4, 32, False),
                                   (1, 9, 128, 8, 8, True), (1, 3, 512, 2, 64, True), (1, 2, 1100, 2, 32, False)],
                          ids=lambda c: "-".join(map(str, c)))
-def test_slot_attention_matches_the_dense_per_head_call(case):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_slot_attention_matches_the_dense_per_head_call(case, dtype):
     """Q, K, V and the gate as slots of one [B,S,N,W,H,D] tensor (what one stacked projection GEMM produces),
     outputs and gradients in slots of buffers of that shape: bit for bit what the per-head call gives on dense
     copies of the slots, with the gradient arriving elsewhere (copied into its slot) and written into the slot."""
@@ -253,10 +254,10 @@ def test_slot_attention_matches_the_dense_per_head_call(case):
     W = 4 if gated else 3
     dev = torch.device("cuda", torch.cuda.current_device())
     g = torch.Generator().manual_seed(13)
-    P = torch.randn((B, S, N, W, H, D), generator=g).to(torch.bfloat16).to(dev).requires_grad_()
-    bias = (torch.randn((1, 1, H, N, N), generator=g) * 0.5).to(torch.bfloat16).to(dev).requires_grad_()
+    P = torch.randn((B, S, N, W, H, D), generator=g).to(dtype).to(dev).requires_grad_()
+    bias = (torch.randn((1, 1, H, N, N), generator=g) * 0.5).to(dtype).to(dev).requires_grad_()
     mask = torch.where(torch.rand((B, S, 1, 1, N), generator=g) < 0.9, 0.0, -1e9).to(dev)
-    dO = torch.randn((B, S, N, H, D), generator=g).to(torch.bfloat16).to(dev)
+    dO = torch.randn((B, S, N, H, D), generator=g).to(dtype).to(dev)
 
     parts = [P.detach()[:, :, :, i].contiguous().requires_grad_() for i in range(W)]
     b2 = bias.detach().clone().requires_grad_()
