@@ -175,3 +175,23 @@ def test_block_projections_of_one_input_match_torch():
         assert torch.equal(a, c)
     for a, c in zip(got, want):
         assert a.shape == c.shape and (a - c).abs().max().item() <= 1e-4 * max(1.0, c.abs().max().item())
+
+
+@pytest.mark.parametrize("with_gate_bias", [True, False])
+def test_block_stacked_projection_matches_torch(with_gate_bias):
+    """Q, K, V and gate as one GEMM with the weights stacked: the result holds the four layers' outputs side by
+    side, and the gradients of the input, of each weight and of the gate's bias are torch's."""
+    from evoformer_triton_amd import block
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((2, 8, 256, 48), generator=g, requires_grad=True)
+    ws = [torch.randn((32, 48), generator=g, requires_grad=True) for _ in range(4)]
+    bg = torch.randn((32,), generator=g, requires_grad=True) if with_gate_bias else None
+    dp = torch.randn((2, 8, 256, 4 * 32), generator=g)
+    leaves = [x] + ws + ([bg] if with_gate_bias else [])
+    want_y = torch.cat([torch.nn.functional.linear(x, w, bg if i == 3 else None) for i, w in enumerate(ws)], -1)
+    want = torch.autograd.grad(want_y, leaves, dp)
+    got_y = block._StackedProjection.apply(x, bg, *ws)
+    got = torch.autograd.grad(got_y, leaves, dp)
+    assert got_y.shape == want_y.shape and (got_y - want_y).abs().max().item() <= 1e-5
+    for a, c in zip(got, want):
+        assert a.shape == c.shape and (a - c).abs().max().item() <= 1e-4 * max(1.0, c.abs().max().item())
