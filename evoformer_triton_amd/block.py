@@ -8,8 +8,13 @@ hipBLASLt on ROCm; the weight gradients are summed over slices of the rows, whic
 GEMMs would leave most of the chip idle) and this package's LayerNorm kernels, and lays the
 results out so that the attention kernels read them as they fall:
 
-  * Q, K, V and the gate come out of four Linear layers as [B,S,N,H*D], which viewed as
-    [B,S,N,H,D] is the per-head ("ds4sci") layout of the kernels: no permute, no copy;
+  * in 16-bit on the GPU Q, K, V and the gate come out of one GEMM with the four weights stacked,
+    as [B,S,N,4*H*D]; viewed as [B,S,N,4,H,D] each is a slot that the kernels take by its strides
+    (per-head rows, a token's 4*H*D elements from the next token's): no permute, no copy, and the
+    gradients come back in the same arrangement, so the projection's backward is one GEMM for the
+    input and one for the weights (`evoformer._SlotAttention`);
+  * elsewhere (fp32, under the tracer, head dims that need padding) they come out of the four
+    Linear layers as [B,S,N,H*D], which viewed as [B,S,N,H,D] is the per-head ("ds4sci") layout;
   * the gate is applied in the forward kernel's epilogue and its gradient comes from the
     backward (`evoformer_attention(..., gate=g)`), so sigmoid(g) * O never makes a round trip
     of its own;
