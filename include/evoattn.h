@@ -31,7 +31,8 @@
 extern "C" {
 #endif
 
-#define EVOATTN_VERSION 2   /* 2: gate, o_gated, dgate appended to EvoAttnParams */
+#define EVOATTN_VERSION 3   /* 2: gate, o_gated, dgate appended to EvoAttnParams; 3: LayerNorm and column-sum entry points,
+                               EVO_FLAG_GATE_DOUT_INPLACE, a gate on a q-family with gaps (slots of a wider buffer) */
 
 /* element types */
 enum {

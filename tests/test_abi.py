@@ -28,7 +28,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert set(names) == set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.evoattn_version() == 2
+    assert lib.evoattn_version() == 3
 
 
 def test_struct_layout_matches_header():
