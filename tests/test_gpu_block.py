@@ -295,3 +295,53 @@ def test_block_takes_the_slot_path_on_the_gpu():
     for a, b in zip(new, old):
         rel = ((a.float() - b.float()).norm() / b.float().norm().clamp_min(1e-12)).item()
         assert rel <= 2e-2 or (a.float() - b.float()).abs().max().item() <= 2e-4, rel
+
+
+def test_slot_attention_random_sweep():
+    """Seeded random shapes (row lengths either side of the kernels' boundaries, every head dim, both 16-bit
+    dtypes, masks, bias dtypes, spare slots): the slot path gives the dense per-head call's bits for the output
+    and every gradient, and leaves spare slots of the gradient zero."""
+    import random
+    import evoformer_triton_amd.evoformer as E
+    r = random.Random(5)
+    dev = torch.device("cuda", torch.cuda.current_device())
+    edges = [1, 7, 32, 33, 64, 100, 128, 129, 200, 256, 257, 320, 384, 385, 512, 513, 640, 768, 769, 1024, 1100, 2048, 2100]
+    for idx in range(60):
+        while True:
+            N, D = r.choice(edges), r.choice([8, 16, 32, 32, 64, 128])
+            S = r.choice([1, 2, 3, 4, 5, 8, 9, 16, 33, 64, 65, 130])
+            B, H = r.choice([1, 1, 2]), r.choice([1, 2, 3, 4, 8])
+            if B * H * S * N * N <= 4.0e7:
+                break
+        dt = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        gated = r.random() < 0.6
+        W = r.choice([4, 4, 5]) if gated else r.choice([3, 3, 4])
+        mask_kind, bias_kind, bias_grad = r.choice(["add", "bool", None]), r.choice(["q", "q", "f32", None]), r.random() < 0.75
+        case = (idx, B, S, N, W, H, D, dt, gated, mask_kind, bias_kind, bias_grad)
+        print("case", case, flush=True)
+        g = torch.Generator().manual_seed(5000 + idx)
+        P = (torch.randn((B, S, N, W, H, D), generator=g) * 0.7).to(dt).to(dev).requires_grad_()
+        bias = None
+        if bias_kind:
+            bias = (torch.randn((r.choice([1, B]), 1, H, N, N), generator=g) * 0.5).to(dt if bias_kind == "q" else torch.float32).to(dev)
+            bias.requires_grad_(bias_grad)
+        mask = None
+        if mask_kind == "add":
+            mask = torch.where(torch.rand((B, S, 1, 1, N), generator=g) < 0.9, 0.0, -1e9).to(dev)
+        elif mask_kind == "bool":
+            mask = (torch.rand((B, S, 1, 1, N), generator=g) < 0.9).to(dev)
+        dO = torch.randn((B, S, N, H, D), generator=g).to(dt).to(dev)
+        parts = [P.detach()[:, :, :, i].contiguous().requires_grad_() for i in range(4 if gated else 3)]
+        b2 = None if bias is None else bias.detach().clone().requires_grad_(bias.requires_grad)
+        ref = E.evoformer_attention(parts[0], parts[1], parts[2], mask, b2, layout="ds4sci", gate=parts[3] if gated else None)
+        with_bias = b2 is not None and b2.requires_grad
+        ref_g = torch.autograd.grad(ref, parts + ([b2] if with_bias else []), dO)
+        out, _ = E._SlotAttention.apply(P, mask, bias, gated)
+        got = torch.autograd.grad(out, [P] + ([bias] if with_bias else []), dO)
+        assert torch.equal(out, ref), case
+        for i in range(len(parts)):
+            assert torch.equal(got[0][:, :, :, i], ref_g[i]), (case, i)
+        for i in range(len(parts), W):
+            assert not got[0][:, :, :, i].any().item(), (case, i)
+        if with_bias:
+            assert torch.equal(got[1], ref_g[len(parts)]), case
