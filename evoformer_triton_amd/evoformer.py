@@ -653,6 +653,16 @@ class _SlotAttention(torch.autograd.Function):
         return DP, dmask, dbias, None
 
 
+def slot_attention(P, res_mask=None, pair_bias=None, gated: bool = False):
+    """Per-head attention on the result of one stacked projection: P [B,S,N,W,H,D] contiguous holds Q, K, V (and,
+    with `gated`, the gate's logits) as its slots 0, 1, 2 (and 3) along W; nothing is copied out of it.  Returns
+    (out, grad_slot): `out` [B,S,N,H,D] is sigmoid(gate) * O (or O), a view whose rows lie W*H*D apart (as a
+    [B*S*N, H*D] matrix it is a GEMM operand as it lies), and `grad_slot` is a view of the same kind that a consumer
+    may write the gradient of `out` into to save its copy.  The gradient of P comes back whole, so the
+    projection's backward is one GEMM for its input and one for its weights."""
+    return _SlotAttention.apply(P, res_mask, pair_bias, bool(gated))
+
+
 def evoformer_attention(Q, K, V, res_mask=None, pair_bias=None, layout: str = "reference", gate=None):
     """Functional form; layout "reference" (flat reshape) or "ds4sci" (per-head permute).
     With `gate` (logits shaped like Q) the result is sigmoid(gate) * O, formed in the forward
