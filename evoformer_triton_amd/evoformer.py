@@ -603,6 +603,7 @@ class _SlotAttention(torch.autograd.Function):
         ctx.bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
         out, grad_slot = OB[:, :, :, 1 if gated else 0], raw[:, :, :, 2]
         ctx.mark_non_differentiable(grad_slot)
+        ctx.set_materialize_grads(False)      # (no tensor of zeros for the second output's gradient, which nobody has)
         return out, grad_slot
 
     @staticmethod
@@ -621,6 +622,8 @@ class _SlotAttention(torch.autograd.Function):
         mask_kind, mstr, mask_orig = ctx.mask_meta
         bias_dt, bstr, bias_orig = ctx.bias_meta
         slot = OB[:, :, :, 2]
+        if dout is None:                      # the output took no part in what is differentiated
+            return torch.zeros_like(P), None, None, None
         in_place = dout.data_ptr() == slot.data_ptr() and dout.dtype == slot.dtype and dout.shape == slot.shape and all(
             n == 1 or a == b for n, a, b in zip(slot.shape, dout.stride(), slot.stride()))
         if not in_place:
