@@ -345,3 +345,23 @@ def test_slot_attention_random_sweep():
             assert not got[0][:, :, :, i].any().item(), (case, i)
         if with_bias:
             assert torch.equal(got[1], ref_g[len(parts)]), case
+
+
+def test_block_forward_without_autograd():
+    """Serving: under no_grad, under inference_mode and with frozen parameters the block's forward gives the
+    training forward's bits."""
+    from evoformer_triton_amd.block import GatedAttentionBlock
+    dev = torch.device("cuda", torch.cuda.current_device())
+    torch.manual_seed(2)
+    blk = GatedAttentionBlock(64, 32, 4, c_z=32).to(dev).to(torch.bfloat16)
+    m = torch.randn(1, 6, 128, 64, device=dev).to(torch.bfloat16)
+    z = torch.randn(1, 128, 128, 32, device=dev).to(torch.bfloat16)
+    mask = (torch.rand(1, 6, 128, device=dev) < 0.9).float()
+    ref = blk(m, z, mask).detach()
+    with torch.no_grad():
+        assert torch.equal(blk(m, z, mask), ref)
+    with torch.inference_mode():
+        assert torch.equal(blk(m, z, mask), ref)
+    for p in blk.parameters():
+        p.requires_grad_(False)
+    assert torch.equal(blk.eval()(m, z, mask), ref)
