@@ -295,6 +295,18 @@ def block_bench(profile_steps=0):
             row[name] = {"eager_us": round(timeit(step, 20), 1), "graph_replay_us": round(timeit(graph.replay, 20), 1),
                          "peak_bytes_beyond_inputs": int(peak)}
             del graph
+
+            def forward_only():
+                with torch.no_grad():
+                    return fwd(m, z, mask)
+            forward_only()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                forward_only()
+            row[name]["forward_only_eager_us"] = round(timeit(forward_only, 20), 1)
+            row[name]["forward_only_graph_replay_us"] = round(timeit(graph.replay, 20), 1)
+            del graph
         rows.append(row)
     print(json.dumps({"block": {"what": "GatedAttentionBlock forward + backward, bf16, one MI355X", "rows": rows}}))
 
