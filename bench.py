@@ -77,7 +77,7 @@ def parse():
                     help="instead of the step benchmark: forward + backward of the gated row-attention block around "
                          "the kernels (LayerNorm, projections, pair-bias projection, attention with the gate, output "
                          "projection) beside the same block in plain torch operations, eager and replayed from a graph, "
-                         "as one JSON line")
+                         "and the forward alone without autograd, as one JSON line")
     ap.add_argument("--block-profile", action="store_true",
                     help="--steps eager steps of the block through the kernels at C2's shape (S=512, N=256, H=8, D=32, "
                          "c_m=256, c_z=128) and nothing else: the run to put under rocprofv3 --kernel-trace")
