@@ -53,6 +53,12 @@ struct FwdRingGeo {
     static __device__ __forceinline__ int swz(int r, int c) { return r * (D * 2) + ((c ^ ((r / RPB) % C)) << 4); }
 };
 
+// The gated form's copy of the gate logits in LDS: per wave its 32 query rows of D 16-bit values, in pieces of
+// 64 lanes x 16 bytes (at head dim 8 half a piece holds them).
+template <int D> constexpr int kGatePieces = D >= 16 ? D / 16 : 1;
+template <int D> constexpr int kGateWaveBytes = kGatePieces<D> * 1024;
+template <int D> constexpr int kGateBytes = 8 * kGateWaveBytes<D>;
+
 // Workgroup barrier that orders LDS traffic only: the loads of the next row and the stores
 // of the last one stay in flight across it (__syncthreads() would wait for them).
 __device__ __forceinline__ void lds_barrier_f() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -87,8 +93,9 @@ static __host__ __device__ inline bool fwdr_rows16(const EvoAttnParams &p) {
 }
 
 // BIASK: 0 no bias, 1 fp32 tiles (x log2(e), accumulator order) as C operands, 2 the caller's 16-bit rows through the identity
-// GATED: the output gate in the epilogue (a kernel of its own: the ungated one carries none of its registers)
-template <typename T, int D, int BIASK, bool GATED>
+// GATED: the output gate in the epilogue (kernels of their own: the ungated one carries none of their registers);
+// 1: the gate's logits asked for in the epilogue, 2: copied into LDS while the row is computed (see gate_dma below)
+template <typename T, int D, int BIASK, int GATED>
 __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     typedef FwdRingGeo<D> R;
     constexpr int C = R::C;
@@ -198,6 +205,14 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     if (nrows <= 0) return;   // uniform over the workgroup
     // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
+    // where the gated form's copy of the gate logits lies: behind the stages (and the bias rows' copy where that is used)
+    constexpr int kStageMost = BIASK == 2 && R::LDS_BYTES < kBiasCopyBytes ? kBiasCopyBytes : R::LDS_BYTES;
+    const int gate_off = BIASK == 2 && !fwdr_rows16(p) ? kStageMost : R::LDS_BYTES;
+    // Taken where a head's rows lie apart (heads inside a token: 8-byte pieces of 2 D bytes out of every row of
+    // the tensor; gated forward at S = 512, N = 256, H = 8, head dim 32: 144 against 157 us); where they lie one
+    // after the other the loads from the epilogue are as fast or faster (133 against 137 us).  Two kernels: one
+    // kernel with both ways spills more and runs the second case at 144 us.
+    constexpr bool gate_dma = GATED == 2;
 
     // ---- the stage of row s_begin + t lives in buffer t & 1.  It is a list of 1 KB pieces
     // (64 lanes x 16 bytes): K, V, then the mask columns; piece n belongs to wave n % 8.  Lane
@@ -280,6 +295,22 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         EVO_TR(1);
         EVO_TR(2);
         const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+        if constexpr (GATED) {
+            // The gate logits of the wave's own 32 query rows go to LDS by the load path itself (16 bytes per lane,
+            // lane L to L * 16 of the wave's piece, no register in between) while the row is computed: asked for in
+            // the epilogue they were waited for with nothing else to do, and asked for earlier into registers they
+            // cost registers the kernel does not have.  The wave alone writes and reads its piece.
+            if (qact && gate_dma) {
+#pragma unroll
+                for (int i = 0; i < kGatePieces<D>; ++i) {
+                    const int L = i * 64 + lane, row = min(L / C, 31), ch = L % C;
+                    const T *src = (const T *)p.gate + base0 + (int64_t)t * p.stride_s + (int64_t)min(q0 + row, p.N - 1) * sn + ch * 8;
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                                     (__attribute__((address_space(3))) void *)(lds + gate_off + wave * kGateWaveBytes<D> + i * 1024),
+                                                     16, 0, 0);
+                }
+            }
+        }
 
         // m: the maximum the probabilities are relative to; mf: what the mask k-step currently
         // subtracts inside the MFMA (m, or 0 while m is not yet known or too large to be
@@ -522,9 +553,14 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                     for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
                         for (int r = 0; r < 16; ++r) oacc[dt][r] *= inv;
-                        // (asked for here and not ahead of the row's stores: eight more registers across the
-                        // stash cost the kernel 7 more spilled registers and 14 us, 150 against 136 us)
-                        gate_row_tile<T>((const T *)p.gate + off, dt * 32, D, oacc[dt], g);
+                        // the wave's piece of the gate, in LDS since the top of the row (the compiler does not
+                        // order the reads after that copy by itself)
+                        if (gate_dma) {
+                            if (dt == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                            gate_row_tile<T>((const T *)(lds + gate_off + wave * kGateWaveBytes<D>) + li * D, dt * 32, D, oacc[dt], g);
+                        } else {
+                            gate_row_tile<T>((const T *)p.gate + off, dt * 32, D, oacc[dt], g);
+                        }
                         store_row_tile<T>((T *)p.o_gated + off, dt * 32, D, oacc[dt], 1.0f, g);
                     }
                 }
@@ -537,15 +573,15 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, int BIASK, bool GATED>
+template <typename T, int D, int BIASK, int GATED>
 static int fwdr_launch_g(const EvoAttnParams &p, const Extra &e0, hipStream_t st) {
     typedef FwdRingGeo<D> R;
     static PerDevice done{};
     int cus = 256;
     auto kern = mfma_fwd_ring<T, D, BIASK, GATED>;
     constexpr int LDS_MOST = BIASK == 2 && R::LDS_BYTES < kBiasCopyBytes ? kBiasCopyBytes : R::LDS_BYTES;
-    if (const int rc = ensure_dynamic_lds((const void *)kern, LDS_MOST, done, &cus)) return rc;
-    const int lds_bytes = BIASK == 2 && !fwdr_rows16(p) ? LDS_MOST : R::LDS_BYTES;
+    if (const int rc = ensure_dynamic_lds((const void *)kern, LDS_MOST + (GATED == 2 ? kGateBytes<D> : 0), done, &cus)) return rc;
+    const int lds_bytes = (BIASK == 2 && !fwdr_rows16(p) ? LDS_MOST : R::LDS_BYTES) + (GATED == 2 ? kGateBytes<D> : 0);
     // one workgroup per CU: chunks of S rows such that (b, h, chunk) items about fill the chip
     Extra e = e0;
     const int bh = p.B * p.H;
@@ -559,7 +595,8 @@ static int fwdr_launch_g(const EvoAttnParams &p, const Extra &e0, hipStream_t st
 
 template <typename T, int D, int BIASK>
 static int fwdr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    return p.gate ? fwdr_launch_g<T, D, BIASK, true>(p, e, st) : fwdr_launch_g<T, D, BIASK, false>(p, e, st);
+    if (!p.gate) return fwdr_launch_g<T, D, BIASK, 0>(p, e, st);
+    return p.stride_h < p.stride_n ? fwdr_launch_g<T, D, BIASK, 2>(p, e, st) : fwdr_launch_g<T, D, BIASK, 1>(p, e, st);
 }
 
 // whether the form with resident fp32 bias tiles keeps them in registers (the dispatch in api.hip sends an
