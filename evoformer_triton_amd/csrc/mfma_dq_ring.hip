@@ -20,12 +20,15 @@
 // here, `global_load_lds_dwordx4` moves about 16 bytes per clock and CU and holds up the
 // other waves' LDS reads while it does, a microsecond per S row; a 16-byte `ds_write` per
 // lane does not.
+#include <type_traits>
+
 #include "bwd_common.h"
 #include "kernels.h"
 
 #ifndef EVO_D
 #error "compile with -DEVO_D=<head dim>"
 #endif
+
 
 namespace evo {
 
@@ -47,13 +50,14 @@ struct RingGeo {
     static constexpr int TPW = TPB / KQ;                     // key tiles per stage and wave
     static constexpr int QR = 32 * QT;                       // query rows per workgroup
     static constexpr int DP = (D + 31) / 32 * 32;
-    static constexpr int RP = DP + 4;                        // pitch of a partial dQ row (floats)
+    static constexpr int RP = DP;                            // pitch of a partial dQ row (floats); 16-byte pieces swizzled by row
     static constexpr int K_BYTES = BKV * D * 2;
-    static constexpr int A_BYTES = BKV * 16;
+    static constexpr int A_BYTES = BKV * 16;                 // the mask operand chunks as they lie in memory
+    static constexpr int A_LDS = BKV * 8;                    // and in the stage: the three mask columns (hi, mid, lo, 0) alone
     static constexpr int Q_BYTES = QR * D * 2;
     static constexpr int OFF_V = K_BYTES;
     static constexpr int OFF_A = 2 * K_BYTES;
-    static constexpr int OFF_Q = OFF_A + A_BYTES;
+    static constexpr int OFF_Q = OFF_A + A_LDS;
     static constexpr int OFF_G = OFF_Q + Q_BYTES;
     static constexpr int OFF_O = OFF_G + Q_BYTES;
     static constexpr int OFF_L = OFF_O + Q_BYTES;                   // -log2-sum-exp of the QR query rows as (hi, mid, lo, 0)
@@ -61,10 +65,15 @@ struct RingGeo {
     static constexpr int RED_BYTES = 8 * 32 * RP * 4;
     static constexpr int STAGE_1K = (STAGE_BYTES + 1023) / 1024 * 1024;
     // The partial dQ tiles get LDS of their own where 160 KB allow it; otherwise they lie in the
-    // buffer of the stage just consumed.
+    // buffer of the stage just consumed.  Where two such areas fit, the rows alternate between
+    // them and a row needs no barrier between its tiles and the write of its partials.
     static constexpr bool OWN_RED = 2 * STAGE_1K + RED_BYTES <= 160 * 1024;
+    static constexpr bool TWO_RED = 2 * STAGE_1K + 2 * RED_BYTES <= 160 * 1024;
     static constexpr int BUF_BYTES = OWN_RED ? STAGE_1K : ((STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES) + 1023) / 1024 * 1024;
-    static constexpr int LDS_BYTES = OWN_RED ? 2 * BUF_BYTES + RED_BYTES : 2 * BUF_BYTES;
+    static constexpr int LDS_BYTES = TWO_RED ? 2 * BUF_BYTES + 2 * RED_BYTES : OWN_RED ? 2 * BUF_BYTES + RED_BYTES : 2 * BUF_BYTES;
+    // float offset of the 16-byte piece c4 of row r inside a partial dQ area (pieces XOR-swizzled by row: a
+    // wave's 16-byte writes and the 16-byte reads of the sum both spread over all banks at a pitch of DP floats)
+    static __device__ __forceinline__ int red_at(int r, int c4) { return r * RP + ((c4 ^ (r & 7)) << 2); }
     // 1 KB pieces (64 lanes x 16 bytes) per segment of a stage
     static constexpr int I_K = K_BYTES / 1024, I_A = A_BYTES / 1024, I_Q = Q_BYTES / 1024;
     static constexpr int I_KVA = 2 * I_K + I_A;
@@ -78,10 +87,12 @@ struct RingGeo {
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 #ifdef EVO_TRACE
+// a cycle count per phase and wave for EVO_TRACE_ROWS rows of every workgroup's chunk, from its ninth row on
+#define EVO_TRACE_ROWS 8
 #define EVO_TR(slot)                                                                             \
     do {                                                                                         \
-        if (e.trace && (threadIdx.x & 63) == 0 && s == s_begin + 3)                              \
-            e.trace[((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (slot)] = wall_clock64(); \
+        if (e.trace && (threadIdx.x & 63) == 0 && s >= s_begin + 8 && s < s_begin + 8 + EVO_TRACE_ROWS)   \
+            e.trace[(((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * EVO_TRACE_ROWS + (s - s_begin - 8)) * 16 + (slot)] = clock64(); \
     } while (0)
 #else
 #define EVO_TR(slot) do {} while (0)
@@ -161,8 +172,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // piece m of a row-major block fills LDS slot 64 m + i of that block, which the swizzle
     // assigns to some chunk of some row.
     constexpr int IPW = (R::I_ALL + 7) / 8;   // most pieces one wave moves per stage
-    u32x4 stg[IPW];
-    float lse_stg = 0.0f;
+    struct Staged {
+        u32x4 v[IPW];
+        float lse;
+    };
     // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
     // Where piece n of key block blk comes from and goes to: a base that every lane shares for
@@ -181,7 +194,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             d.base = reinterpret_cast<const unsigned char *>(e.m2a + ((int64_t)b * p.S + s_begin) * np256 + blk * BKV + m * 64);
             d.row_step = (int64_t)np256 * 16;
             d.lane_off = lane * 16u;
-            d.dst = R::OFF_A + m * 1024;
+            d.dst = R::OFF_A + m * 512;
         } else {
             const T *base;
             int m, row0, off;
@@ -210,23 +223,47 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     }
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
+    // With one stage per row a piece's address is a pointer that all lanes share, advanced by the
+    // scalar unit from row to row, plus a 32-bit lane offset that never changes: no 64-bit
+    // multiplication per piece and row.  `fnext` is the row the pointers stand at.
+    const unsigned char *fptr[NBLK == 1 ? IPW : 1];
+    const float *flse = p.lse + ((int64_t)bh * p.S + s_begin) * p.N;   // of the row the pointers stand at
+    const unsigned flse_off = (unsigned)min(qbase + lane, p.N - 1);
+    if (NBLK == 1) {
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) fptr[i] = fixed[i].base;
+    }
+    // moves the pointers from stage t to stage t + 1 (they stay at the last stage)
+    auto fetch_advance = [&](int t) {
+        if (NBLK != 1 || t + 1 > T_total - 1) return;
+#pragma unroll
+        for (int i = 0; i < IPW; ++i) fptr[i] += fixed[i].row_step;
+        flse += p.N;
+    };
     // pieces [i0, i1) of stage t; the last piece takes the log-sum-exp along
-    auto fetch_part = [&](int t, int i0, int i1) {
+    auto fetch_part = [&](Staged &stg, int t, int i0, int i1) {
         t = min(t, T_total - 1);
         const int row = t / NBLK, blk = t % NBLK;
         const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             if (i < i0 || i >= i1) continue;
-            const Piece d = NBLK == 1 ? fixed[i] : describe(min(wave + 8 * i, ninst - 1), blk);
-            stg[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
+            if (NBLK == 1) {
+                stg.v[i] = *reinterpret_cast<const u32x4 *>(fptr[i] + fixed[i].lane_off);
+            } else {
+                const Piece d = describe(min(wave + 8 * i, ninst - 1), blk);
+                stg.v[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
+            }
         }
         // the log-sum-exp of the slab's rows travels the same way (one value per lane; every
         // wave asks, wave 0 stores): a load whose result is carried into the next row's
         // prologue in a register would make that prologue wait for everything requested here
-        if (i1 >= IPW) lse_stg = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
+        if (i1 >= IPW) {
+            if (NBLK == 1) stg.lse = flse[flse_off];
+            else stg.lse = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
+        }
     };
-    auto fetch = [&](int t) { fetch_part(t, 0, IPW); };
+    auto fetch = [&](Staged &stg, int t) { fetch_part(stg, t, 0, IPW); };
     constexpr int SPLIT = IPW / 2;   // pieces asked for at the top of a row; the rest after its prologue
     // What every wave of a query tile would otherwise redo in its prologue is done once, by
     // the wave that writes the piece: Q goes to LDS scaled by scale*log2(e) (where the scaled
@@ -234,10 +271,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // for a row with every key masked, and the log-sum-exp as its three operand columns.
     constexpr bool PRESCALE = !G::RESID;
     bool stage_dead = PRESCALE && uniform_load(e.dead + b * p.S + s_begin) != 0;
-    auto stash_part = [&](int t, int i0, int i1) {
+    auto stash_part = [&](const Staged &stg, int t, int i0, int i1, int par) {   // par: the buffer of stage t, t & 1
         const int blk = t % NBLK;
         const int ninst = t >= T_total ? 0 : blk == 0 ? R::I_ALL : R::I_KVA;
-        unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+        unsigned char *buf = lds + par * R::BUF_BYTES;
         const float cq = stage_dead ? 0.0f : cs;   // (the flag of the row this stage belongs to)
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
@@ -245,52 +282,85 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             const int n = wave + 8 * i;
             if (n < ninst) {
                 const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
-                if (PRESCALE && n >= R::I_KVA && n < R::I_KVA + R::I_Q)
-                    *reinterpret_cast<v8 *>(buf + dst + lane * 16) = scaled8<T>(__builtin_bit_cast(v8, stg[i]), cq);
+                if (n >= 2 * R::I_K && n < R::I_KVA)   // of a mask chunk (hi, mid, lo, 1, 1, 1, 0, 0) the first 8 bytes
+                    *reinterpret_cast<uint2 *>(buf + dst + lane * 8) = make_uint2(stg.v[i][0], stg.v[i][1]);
+                else if (PRESCALE && n >= R::I_KVA && n < R::I_KVA + R::I_Q)
+                    *reinterpret_cast<v8 *>(buf + dst + lane * 16) = scaled8<T>(__builtin_bit_cast(v8, stg.v[i]), cq);
                 else
-                    *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg[i];
+                    *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg.v[i];
             }
         }
         if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR)
-            *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-lse_stg * kLog2e);
+            *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-stg.lse * kLog2e);
     };
-    auto stash = [&](int t) { stash_part(t, 0, IPW); };
+    auto stash = [&](const Staged &stg, int t, int par) { stash_part(stg, t, 0, IPW, par); };
 
-    // The partial dQ^T tiles of a query tile (one per wave that works on it, fp32, in the buffer of the
-    // stage they came from) summed, scaled and stored as row `base` of dQ.
-    auto sum_store = [&](const float *red, int64_t base) {
-        T *dQ = (T *)p.dq + base;
-        for (int it = tid; it < QR * (D / 4); it += 512) {
-            const int q = it / (D / 4), d4 = (it % (D / 4)) * 4;
-            const int w0 = (q >> 5) * KQ, ql = q & 31;
-            f32x4 sum = *reinterpret_cast<const f32x4 *>(&red[(w0 * 32 + ql) * RP + d4]);
+    // The partial dQ^T tiles of a query tile (one per wave that works on it, fp32) summed, scaled and stored as a
+    // row of dQ.  The older wave of every SIMD (waves 0..3), which the issue arbitration favours and which would
+    // otherwise wait at the next barrier for the younger one, does the sums: thread i of those 256 takes the
+    // 16-byte pieces i, i + 256, ... of the slab's QR x D results.  What does not depend on the row is formed once.
+    constexpr int NSUM = QR * (D / 4), NIT = (NSUM + 255) / 256;
+    int sum_lds[NIT];         // float offset of the first wave's partial inside a partial dQ area
+    unsigned sum_goff[NIT];   // byte offset of the piece from the first query row of the problem in dQ
+    bool sum_ok[NIT];
 #pragma unroll
-            for (int w = 1; w < KQ; ++w) sum += *reinterpret_cast<const f32x4 *>(&red[((w0 + w) * 32 + ql) * RP + d4]);
-            if (qbase + q < p.N)
-                store4<T>(dQ + (int64_t)(qbase + q) * sn + d4, sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
+    for (int j = 0; j < NIT; ++j) {
+        const int it = (tid & 255) + 256 * j;
+        const int q = min(it / (D / 4), QR - 1), d4 = (it % (D / 4)) * 4;
+        sum_lds[j] = R::red_at((q >> 5) * KQ * 32 + (q & 31), d4 >> 2);
+        sum_goff[j] = (unsigned)(min(qbase + q, p.N - 1) * (int)sn + d4) * 2u;
+        sum_ok[j] = it < NSUM && qbase + q < p.N;
+    }
+    // `row` points at the problem's first row in dQ (shared by the lanes)
+    auto sum_store = [&](const float *red, unsigned char *row) {
+        if (wave >= 4) return;
+        f32x4 part[NIT][KQ];
+#pragma unroll
+        for (int j = 0; j < NIT; ++j)
+#pragma unroll
+            for (int w = 0; w < KQ; ++w) part[j][w] = *reinterpret_cast<const f32x4 *>(&red[sum_lds[j] + w * 32 * RP]);
+#pragma unroll
+        for (int j = 0; j < NIT; ++j) {
+            f32x4 sum = part[j][0];
+#pragma unroll
+            for (int w = 1; w < KQ; ++w) sum += part[j][w];
+            if (sum_ok[j])
+                store4<T>(reinterpret_cast<T *>(row + sum_goff[j]), sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
                           sum[3] * p.scale);
         }
     };
+    unsigned char *dq_row = reinterpret_cast<unsigned char *>((T *)p.dq + base0);   // of the row whose partials are summed next
     // The sum of a row's partials waits until the next row's first stage barrier has been
     // passed: nobody writes where the partials lie before another barrier has followed, which
     // with several key blocks per row is the next stage barrier and with one is a barrier of
     // its own (XBAR) between the row's tiles and the write of its partials.
     static_assert(NBLK == 1 || R::OWN_RED, "rows of several key blocks keep the partials out of the stage buffers");
-    constexpr bool XBAR = NBLK == 1;
+    constexpr bool XBAR = NBLK == 1 && !R::TWO_RED;
     // With the partials out of the stage buffers, the buffer of the next stage is free from
     // the stage barrier on: every wave asks for half of its pieces at the top of the row and
     // writes them to LDS between its two tiles, while other waves compute; the other half it
     // asks for after the row's prologue and writes after the tiles.
     constexpr bool MID = NBLK == 1 && R::OWN_RED && TPW >= 2;
-    auto red_of = [&](int stage) { return (float *)(lds + (R::OWN_RED ? 2 * R::BUF_BYTES : (stage & 1) * R::BUF_BYTES)); };
+    // where the partials of the row that ended with stage `stage` lie; par: stage & 1 (one stage per row: the row's parity)
+    auto red_of = [&](int stage, int par) {
+        return (float *)(lds + (R::TWO_RED ? 2 * R::BUF_BYTES + (NBLK == 1 ? par : stage / NBLK & 1) * R::RED_BYTES
+                                : R::OWN_RED ? 2 * R::BUF_BYTES : par * R::BUF_BYTES));
+    };
 
-    fetch(0);
-    stash(0);
+    Staged sa;
+    fetch(sa, 0);
+    fetch_advance(0);
+    stash(sa, 0, 0);
 
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
     int t = 0;
-    for (int s = s_begin; s < s_end; ++s) {
+    // One S row.  With one stage per row the rows are unrolled in pairs, so that which of the two
+    // buffers a row reads (PAR = 0, 1) is known at compile time and every LDS address is a register
+    // that never changes plus an immediate offset; PAR = -1: the stage number decides.
+    auto do_row = [&](const int s, auto par_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        Staged &cur = sa, &nxt = sa;
         const unsigned pid = bh * (unsigned)p.S + s;
         Prob pr;
         pr.b = b; pr.h = h; pr.s = s;
@@ -312,19 +382,23 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 #pragma unroll
         for (int blk = 0; blk < NBLK; ++blk, ++t) {
             EVO_TR(0);
-            EVO_TR(1);
             lds_barrier();   // stage t is in LDS; stage t-1 and the last reduction are done with
-            EVO_TR(2);
+            EVO_TR(1);
             // The CU's load path takes a stage's 48 requests (D = 32) at 16 clocks each: half of
             // them go out now and half after the row's prologue rather than all queue up behind
             // it (where the staging writes cannot be split, the waves take turns instead).  With
             // few requests per wave there is nothing to gain.
             const bool early = !(NBLK == 1 && IPW >= 4) || (wave & 1) == 0;
-            if (MID) fetch_part(t + 1, 0, SPLIT);
-            else if (early) fetch(t + 1);
+            if (MID) fetch_part(nxt, t + 1, 0, SPLIT);
+            else if (early) fetch(nxt, t + 1);
+            EVO_TR(2);
+            const int par = PAR >= 0 ? PAR : (t & 1);
+            buf = lds + par * R::BUF_BYTES;
+            if (blk == 0 && s > s_begin) {
+                sum_store(red_of(t - 1, par ^ 1), dq_row);
+                dq_row += p.stride_s * 2;
+            }
             EVO_TR(3);
-            buf = lds + (t & 1) * R::BUF_BYTES;
-            if (blk == 0 && s > s_begin) sum_store(red_of(t - 1), pr.base - p.stride_s);
 
             if (blk == 0) {
                 // this lane's half of the query row: Q (scaled), dO, and delta = <dO, O>
@@ -363,15 +437,21 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 }
             }
 
-            if (MID) fetch_part(t + 1, SPLIT, IPW);
-            else if (!early) fetch(t + 1);
             EVO_TR(4);
+            if (MID) fetch_part(nxt, t + 1, SPLIT, IPW);
+            else if (!early) fetch(nxt, t + 1);
+            fetch_advance(t + 1);
+            EVO_TR(5);
             {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
                     const int tb = jj * KQ + kq;         // tile inside the stage
                     const int kt = blk * TPB + tb;
-                    if (MID && jj == TPW - 1) stash_part(t + 1, 0, SPLIT);
+                    if (MID && jj == TPW - 1) {
+                        EVO_TR(6);
+                        stash_part(cur, t + 1, 0, SPLIT, par ^ 1);
+                        EVO_TR(7);
+                    }
                     // wave-uniform; no gradient goes through the scores of a row that a bool mask drops
                     // entirely: its tiles are skipped, dQ stays zero and dBias unchanged
                     if (qact && kt < NT && !kill) {
@@ -391,7 +471,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                                 // upper half (lane group 1) is zero on the query side: there the key side may hold
                                 // any finite values, so both lane groups read the same columns and no lane is
                                 // cleared or masked per tile.
-                                ka[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_A + (tb * 32 + li) * 16);  // mask x ones, ones x -lse
+                                ka[ks] = aug8<T>(*reinterpret_cast<const uint2 *>(buf + R::OFF_A + (tb * 32 + li) * 8), one3);  // mask x ones, ones x -lse
                                 va[ks] = aug8<T>(one3, zero3);                                                 // ones x -delta
                             }
                         }
@@ -444,17 +524,18 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     }
                 }
             }
+            EVO_TR(8);
             // into the other buffer, free since the barrier above
-            if (MID) stash_part(t + 1, SPLIT, IPW);
-            else if (R::OWN_RED) stash(t + 1);
+            if (MID) stash_part(cur, t + 1, SPLIT, IPW, par ^ 1);
+            else if (R::OWN_RED) stash(cur, t + 1, par ^ 1);
         }
 
         // Partial dQ^T of this wave: lane = query li, register r = dim dt*32 + crow(r, g).  The
         // waves of a query tile meet in LDS.
-        EVO_TR(5);
+        EVO_TR(9);
         if (XBAR) lds_barrier();
-        EVO_TR(6);
-        float *red = red_of(t - 1);
+        const int lpar = PAR >= 0 ? PAR : ((t - 1) & 1);   // of the row's last stage
+        float *red = red_of(t - 1, lpar);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -462,18 +543,24 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                 f32x4 v;
                 v[0] = dqacc[dt][4 * rr]; v[1] = dqacc[dt][4 * rr + 1];
                 v[2] = dqacc[dt][4 * rr + 2]; v[3] = dqacc[dt][4 * rr + 3];
-                *reinterpret_cast<f32x4 *>(&red[(wave * 32 + li) * RP + dt * 32 + 8 * rr + 4 * g]) = v;
+                *reinterpret_cast<f32x4 *>(&red[R::red_at(wave * 32 + li, dt * 8 + 2 * rr + g)]) = v;
             }
-        EVO_TR(7);
         // where the partials share the stage buffers, the other buffer held the last row's;
         // everyone has summed them by now
-        if (!R::OWN_RED) stash(t);
-        EVO_TR(8);
-        EVO_TR(9);
+        if (!R::OWN_RED) stash(cur, t, lpar ^ 1);
+        EVO_TR(10);
+    };
+    if (NBLK == 1) {
+        for (int s = s_begin; s < s_end; s += 2) {
+            do_row(s, std::integral_constant<int, 0>{});
+            if (s + 1 < s_end) do_row(s + 1, std::integral_constant<int, 1>{});
+        }
+    } else {
+        for (int s = s_begin; s < s_end; ++s) do_row(s, std::integral_constant<int, -1>{});
     }
     if (s_end > s_begin) {
         lds_barrier();
-        sum_store(red_of(t - 1), base0 + (int64_t)(s_end - 1 - s_begin) * p.stride_s);
+        sum_store(red_of(t - 1, (t - 1) & 1), dq_row);
     }
 
     if (want_dbias && qact && q0 + li < p.N) {
