@@ -300,33 +300,39 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // otherwise wait at the next barrier for the younger one, does the sums: thread i of those 256 takes the
     // 16-byte pieces i, i + 256, ... of the slab's QR x D results.  What does not depend on the row is formed once.
     constexpr int NSUM = QR * (D / 4), NIT = (NSUM + 255) / 256;
-    int sum_lds[NIT];         // float offset of the first wave's partial inside a partial dQ area
-    unsigned sum_goff[NIT];   // byte offset of the piece from the first query row of the problem in dQ
-    bool sum_ok[NIT];
+    constexpr int RPP = 256 / (D / 4);          // query rows that one pass of the 256 threads covers
+    // Where a pass covers whole query tiles (head dims up to 32), a thread's pieces are its first one plus a
+    // step that all lanes share, in LDS as in memory: one offset each is kept, not one per piece.
+    constexpr bool AFFINE = RPP % 32 == 0;
+    constexpr int NK = AFFINE ? 1 : NIT;
+    int sum_lds[NK];          // float offset of the first wave's partial inside a partial dQ area
+    unsigned sum_goff[NK];    // byte offset of the piece from the first query row of the problem in dQ
 #pragma unroll
-    for (int j = 0; j < NIT; ++j) {
+    for (int j = 0; j < NK; ++j) {
         const int it = (tid & 255) + 256 * j;
         const int q = min(it / (D / 4), QR - 1), d4 = (it % (D / 4)) * 4;
         sum_lds[j] = R::red_at((q >> 5) * KQ * 32 + (q & 31), d4 >> 2);
-        sum_goff[j] = (unsigned)(min(qbase + q, p.N - 1) * (int)sn + d4) * 2u;
-        sum_ok[j] = it < NSUM && qbase + q < p.N;
+        sum_goff[j] = (unsigned)((qbase + q) * (int)sn + d4) * 2u;
     }
+    const int sum_q0 = qbase + (tid & 255) / (D / 4);   // the query row of the thread's first piece
     // `row` points at the problem's first row in dQ (shared by the lanes)
     auto sum_store = [&](const float *red, unsigned char *row) {
         if (wave >= 4) return;
         f32x4 part[NIT][KQ];
 #pragma unroll
-        for (int j = 0; j < NIT; ++j)
+        for (int j = 0; j < NIT; ++j) {
+            const int o = AFFINE ? sum_lds[0] + j * (RPP / 32) * KQ * 32 * RP : sum_lds[j < NK ? j : 0];
 #pragma unroll
-            for (int w = 0; w < KQ; ++w) part[j][w] = *reinterpret_cast<const f32x4 *>(&red[sum_lds[j] + w * 32 * RP]);
+            for (int w = 0; w < KQ; ++w) part[j][w] = *reinterpret_cast<const f32x4 *>(&red[o + w * 32 * RP]);
+        }
 #pragma unroll
         for (int j = 0; j < NIT; ++j) {
             f32x4 sum = part[j][0];
 #pragma unroll
             for (int w = 1; w < KQ; ++w) sum += part[j][w];
-            if (sum_ok[j])
-                store4<T>(reinterpret_cast<T *>(row + sum_goff[j]), sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale,
-                          sum[3] * p.scale);
+            const bool ok = (tid & 255) + 256 * j < NSUM && sum_q0 + j * RPP < p.N;
+            unsigned char *dst = AFFINE ? row + (int64_t)j * RPP * sn * 2 + sum_goff[0] : row + sum_goff[j < NK ? j : 0];
+            if (ok) store4<T>(reinterpret_cast<T *>(dst), sum[0] * p.scale, sum[1] * p.scale, sum[2] * p.scale, sum[3] * p.scale);
         }
     };
     unsigned char *dq_row = reinterpret_cast<unsigned char *>((T *)p.dq + base0);   // of the row whose partials are summed next

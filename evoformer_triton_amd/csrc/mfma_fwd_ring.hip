@@ -64,10 +64,12 @@ template <int D> constexpr int kGateBytes = 8 * kGateWaveBytes<D>;
 __device__ __forceinline__ void lds_barrier_f() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 #ifdef EVO_TRACE
+// a cycle count per phase and wave for EVO_TRACE_ROWS rows of every workgroup's chunk, from its fifth row on
+#define EVO_TRACE_ROWS 8
 #define EVO_TR(slot)                                                                             \
     do {                                                                                         \
-        if (e.trace && (threadIdx.x & 63) == 0 && t == 3)                                        \
-            e.trace[((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 16 + (slot)] = wall_clock64(); \
+        if (e.trace && (threadIdx.x & 63) == 0 && t >= 4 && t < 4 + EVO_TRACE_ROWS)              \
+            e.trace[(((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * EVO_TRACE_ROWS + (t - 4)) * 16 + (slot)] = clock64(); \
     } while (0)
 #else
 #define EVO_TR(slot) do {} while (0)
@@ -219,56 +221,56 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
     // i of piece m of K or V fills LDS slot 64 m + i of that block, which the swizzle assigns
     // to some chunk of some row.
     u32x4 stg[IPW];
-    // Where a piece comes from and goes to: a base that every lane shares for the first row
-    // of the chunk, its advance per S row (both in bytes), this lane's offset from it, and
-    // the LDS offset inside the stage.  They never change, so they are formed once.
-    struct Piece {
-        const unsigned char *base;
-        int64_t row_step;
-        unsigned lane_off;
-        int dst;
+    // K and V pieces are buffer loads: a resource (in scalar registers) that describes the K or V rows of
+    // the S row asked for next, one lane offset that every K and V piece shares (a piece is 64 / C rows
+    // of C 16-byte chunks; the swizzle depends on the row inside the piece only), and the piece's own
+    // offset, also scalar.  Rows at or beyond N lie past the end of the resource and read as zero (such
+    // keys carry the mask floor), so no lane clamps its row.  The mask columns are padded to 256 keys
+    // and come by plain loads.  In LDS piece n lies at n KB, whatever its kind.
+    static_assert(R::K_BYTES == R::I_K * 1024 && R::OFF_A == 2 * R::I_K * 1024, "piece n of a stage lies at n KB");
+    static_assert(C == 1 || C == 2 || C == 4, "one lane offset for every K and V piece needs a head dim of 8, 16 or 32");
+    const int kv_valid = (int)(((int64_t)(p.N - 1) * sn + D) * 2);   // bytes from a problem's first K (V) row to the end of its last
+    const unsigned kv_voff = (unsigned)((lane / C) * (int)sn * 2 + (((lane % C) ^ (((lane / C) / R::RPB) % C)) << 4));
+    const int kv_piece = (64 / C) * (int)sn * 2;                     // bytes from one K (V) piece to the next
+    // of the row that is asked for next (they stay at the chunk's last row)
+    const unsigned char *krow = reinterpret_cast<const unsigned char *>((const T *)p.k + base0);
+    const unsigned char *vrow = reinterpret_cast<const unsigned char *>((const T *)p.v + base0);
+    const unsigned char *arow = reinterpret_cast<const unsigned char *>(e.m2a + ((int64_t)b * p.S + s_begin) * np256);
+    int frow = 0;
+    auto fetch_row = [&](int t) {   // moves the pointers to row min(t, nrows - 1); t grows by at most one per call
+        if (t > frow && t < nrows) {
+            krow += p.stride_s * 2;
+            vrow += p.stride_s * 2;
+            arow += (int64_t)np256 * 16;
+            frow = t;
+        }
     };
-    Piece pc[IPW];
-#pragma unroll
-    for (int i = 0; i < IPW; ++i) {
-        // (a wave with fewer pieces repeats its last one)
-        const int n = min(wave + 8 * i, R::I_ALL - 1);
-        if (n >= 2 * R::I_K) {
-            const int m = n - 2 * R::I_K;
-            pc[i].base = reinterpret_cast<const unsigned char *>(e.m2a + ((int64_t)b * p.S + s_begin) * np256 + m * 64);
-            pc[i].row_step = (int64_t)np256 * 16;
-            pc[i].lane_off = lane * 16u;
-            pc[i].dst = R::OFF_A + m * 1024;
-        } else {
+    // Loads are unconditional (the row past the end repeats the last row, a wave with fewer pieces
+    // repeats a mask piece) so that the staging registers stay registers.
+    auto fetch_piece = [&](int i) {
+        const int n = wave + 8 * i;   // uniform
+        if (n < 2 * R::I_K) {
             const bool isv = n >= R::I_K;
             const int m = isv ? n - R::I_K : n;
-            const T *base = isv ? (const T *)p.v : (const T *)p.k;
-            const int L = m * 64 + lane;
-            const int r = L / C, cpos = L % C;
-            const int ch = cpos ^ ((r / R::RPB) % C);
-            const int row = min(r, p.N - 1);
-            pc[i].base = reinterpret_cast<const unsigned char *>(base + base0);
-            pc[i].row_step = p.stride_s * 2;
-            pc[i].lane_off = (unsigned)(row * (int)sn + ch * 8) * 2u;
-            pc[i].dst = (isv ? R::OFF_V : 0) + m * 1024;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(isv ? vrow : krow), 0, kv_valid, 0x00020000);
+            stg[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)kv_voff, m * kv_piece, 0);
+        } else {
+            const int m = min(n, R::I_ALL - 1) - 2 * R::I_K;
+            stg[i] = *reinterpret_cast<const u32x4 *>(arow + m * 1024 + lane * 16);
         }
-    }
-    // Loads are unconditional (the row past the end repeats the last row) so that the
-    // staging registers stay registers.
-    auto fetch_piece = [&](int t, int i) {
-        t = min(t, nrows - 1);
-        stg[i] = *reinterpret_cast<const u32x4 *>(pc[i].base + t * pc[i].row_step + pc[i].lane_off);
     };
     auto fetch = [&](int t) {
+        fetch_row(t);
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) fetch_piece(t, i);
+        for (int i = 0; i < IPW; ++i) fetch_piece(i);
     };
+    const int lds_piece0 = wave * 1024 + lane * 16;   // where this lane's 16 bytes of the wave's first piece lie in a stage
     auto stash = [&](int t) {
         if (t >= nrows) return;
-        unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
+        unsigned char *buf = lds + (t & 1) * R::BUF_BYTES + lds_piece0;
 #pragma unroll
         for (int i = 0; i < IPW; ++i)
-            if (wave + 8 * i < R::I_ALL) *reinterpret_cast<u32x4 *>(buf + pc[i].dst + lane * 16) = stg[i];
+            if (wave + 8 * i < R::I_ALL) *reinterpret_cast<u32x4 *>(buf + i * 8192) = stg[i];
     };
     // this lane's half of its query row, straight from global memory
     v8 qraw[KSD], qnext[KSD];
@@ -293,7 +295,6 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         EVO_TR(0);
         lds_barrier_f();   // the stage of this row is in LDS; everybody is done with the row before
         EVO_TR(1);
-        EVO_TR(2);
         const unsigned char *buf = lds + (t & 1) * R::BUF_BYTES;
         if constexpr (GATED) {
             // The gate logits of the wave's own 32 query rows go to LDS by the load path itself (16 bytes per lane,
@@ -483,21 +484,26 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
             f32x16 sa0, sa1;
 #pragma unroll
             for (int step = 0; step < 4; ++step) {
-                EVO_TR(3 + step);
+                EVO_TR(2 + step);
+                // The two waves of a SIMD (w and w + 4) take turns at the higher issue priority, step by
+                // step: left alone the older wave is always served first, ends its row a quarter of a
+                // row early and waits at the barrier while the younger one runs on alone.
+                if (((step ^ (wave >> 2)) & 1) != 0) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
                 {
                     // The next row's requests go out a few per step rather than all after the
                     // barrier: eight waves asking at once queue up behind the CU's load path
                     // (16 clocks per request), and the last in line start their row late.
                     constexpr int PPS = (IPW + 2) / 3;
+                    if (step == 0) fetch_row(t + 1);
 #pragma unroll
                     for (int i = step * PPS; i < (step + 1) * PPS && i < IPW; ++i)
-                        if (step < 3) fetch_piece(t + 1, i);
+                        if (step < 3) fetch_piece(i);
                     if (step == 2) fetch_q(t + 1, qnext);
                 }
                 if (step < nsteps) {  // uniform
                     const float used = mf;
                     scores(step, sa0, sa1);
-                    if (step == 2) EVO_TR(10);
                     v8 pf[4];
                     float ls;
                     // After the first step the scores come out of the MFMA relative to m already
@@ -516,9 +522,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                         settle(step, sa0, sa1, used);
                         probs(sa0, sa1, pf, ls);
                     }
-                    if (step == 2) EVO_TR(11);
                     weigh(step, pf, ls);
-                    if (step == 2) EVO_TR(13);
                 }
             }
 
@@ -530,11 +534,10 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
         // The next stage goes into the other buffer, free since the barrier above.  This comes
         // before the row's own stores: what waits for the staged loads must not have the
         // stores in front of it (vector memory operations complete in order).
-        EVO_TR(8);
+        EVO_TR(6);
         stash(t + 1);
-        EVO_TR(9);
+        EVO_TR(7);
         if (qact) {
-            EVO_TR(7);
             {   // the two lane groups hold the two halves of each query's sum
                 const unsigned u = __float_as_uint(l);
                 auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -566,6 +569,7 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
                 }
             }
         }
+        EVO_TR(8);
 #pragma unroll
         for (int ks = 0; ks < KSD; ++ks) qraw[ks] = qnext[ks];
     }
@@ -620,8 +624,12 @@ static int fwdr_bias(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 int EVO_CAT(mfma_fwdr_max_n_d, EVO_D)() { return EVO_D <= 32 ? 256 : 0; }   // 64: the resident tiles do not fit the registers
 
 int EVO_CAT(launch_mfma_fwdr_d, EVO_D)(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    if (EVO_D > 32) return EVO_EUNSUPPORTED;
+#if EVO_D <= 32
     return p.dtype == EVO_BF16 ? fwdr_bias<bf16_t>(p, e, st) : fwdr_bias<f16_t>(p, e, st);
+#else
+    (void)p; (void)e; (void)st;   // (no kernel is built: the resident bias does not fit the registers at this width)
+    return EVO_EUNSUPPORTED;
+#endif
 }
 
 }  // namespace evo
