@@ -236,7 +236,11 @@ def shape_sweep():
                             (1, 10, 200, 640, 64), (1, 15, 200, 640, 64), (1, 5, 100, 768, 64), (1, 10, 100, 768, 64),
                             (1, 1, 100, 1280, 64), (1, 5, 300, 512, 64), (1, 5, 300, 384, 64)):
         ref.append(one(B, S, N, H, D, "fp32", "reference"))
-    print(json.dumps({"shape_sweep": {"unit": "us; rates in 1e12 scores/s", "rows": rows, "reference_test_shapes": ref}}))
+    print(json.dumps({"shape_sweep": {"unit": "us; rates in 1e12 scores/s",
+                                      "timing": "mean of 20 back-to-back repetitions, no cache flush between them: shapes whose "
+                                                "tensors fit the 256 MB memory-side cache run cache-warm (--reference-sweep "
+                                                "flushes before every repetition, as triton.testing.do_bench does)",
+                                      "rows": rows, "reference_test_shapes": ref}}))
 
 
 def block_bench(profile_steps=0):

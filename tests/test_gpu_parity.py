@@ -22,6 +22,14 @@ pytestmark = pytest.mark.gpu
 BF16_TOL = 2e-2
 # max-abs bound on O, dQ, dK, dV per benchmark configuration
 FULL_TOL = {"C2": BF16_TOL, "C3": BF16_TOL, "C4": BF16_TOL, "C5": BF16_TOL}
+# What the two roundings shared with the reference's kernels (delta from the saved 16-bit output,
+# evoformer.py:313-323; the scaled query operand rounded once from head dim 32 on, :49, :433) cost the
+# gradients that are sums over S rows or over heads and queries, against fp32 eager: the oracle's
+# restatement measured on one MI355X (dBias 1.812e-2 / 4.446e-2 / 4.153e-2 / 2.651e-2, dMask 1.650e-2 /
+# 1.711e-2 / 1.563e-2 / 1.345e-2 for C2 / C3 / C4 / C5) times 1.25.  Constants: the allowance cannot
+# grow with a regression of the forward's output.
+SHARED_ROUNDINGS_CEILING = {"C2": {"dBias": 2.27e-2, "dMask": 2.06e-2}, "C3": {"dBias": 5.56e-2, "dMask": 2.14e-2},
+                            "C4": {"dBias": 5.19e-2, "dMask": 1.95e-2}, "C5": {"dBias": 3.31e-2, "dMask": 1.68e-2}}
 F32_TOL = 1e-5
 GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "*.npz")))
 
@@ -90,6 +98,9 @@ def assert_close(got, ref, tol, names=("O", "dQ", "dK", "dV", "dBias"), what="",
     return errs
 
 
+MODEL_COST_CEILING = 4e-2
+
+
 def assert_close_to_modelled_backward(got, ref, inputs, tol, what, layout="reference"):
     """For inputs that put nearly all of a row's weight on a few keys, whose dK and dV then
     collect hundreds of probabilities each rounded to 16 bits: the gradients are held to `tol`
@@ -97,7 +108,7 @@ def assert_close_to_modelled_backward(got, ref, inputs, tol, what, layout="refer
     of the backward with the roundings the reference's kernels make too (delta from the saved
     output, evoformer.py:313-323; the query operand scaled in the input dtype, :49, :433; P and
     dS cast before the gradient matmuls, :459, :603, :611), and to tol plus that restatement's own
-    distance from fp32 eager against fp32 eager itself."""
+    distance from fp32 eager (at most MODEL_COST_CEILING) against fp32 eager itself."""
     Q, K, V, m, bias, dO = inputs
     D = Q.shape[-1]
     dt = Q.dtype
@@ -107,7 +118,9 @@ def assert_close_to_modelled_backward(got, ref, inputs, tol, what, layout="refer
     assert_close(got, model, tol, names, what=what + " vs the backward from the saved output", round_names=tuple(names))
     for n in names:
         a, b = got[n].detach().float().cpu(), ref[n].detach().float().cpu()
-        cost = (model[n].float() - b).abs().max().item()
+        # (the restatement's own distance, capped: the allowance does not grow without bound; the largest
+        # measured on these inputs is 3.2e-2, dV of rows with one kept key)
+        cost = min((model[n].float() - b).abs().max().item(), MODEL_COST_CEILING)
         bound = tol + cost + half_ulp(torch.maximum(a.abs(), b.abs()), got[n].dtype)
         assert bool(((a - b).abs() <= bound).all()), f"{what} {n}: {(a - b).abs().max().item():.3e} vs fp32 eager (restatement {cost:.3e} away)"
 
@@ -1128,9 +1141,12 @@ def test_benchmark_configs_full_size(E, cfg):
     for n in ("dBias", "dMask"):
         e_f32[n] = max_err(got[n], ref_f32[n])
         e_self[n] = max_err(ref_bf16[n], ref_f32[n])
-        # against fp32 eager itself: what the two shared roundings cost (measured just above) on top
+        # against fp32 eager itself: on top, a constant ceiling on what the two shared roundings cost
+        # (the restatement's own distance, printed below, is held under the same ceiling)
+        ceiling = SHARED_ROUNDINGS_CEILING[cfg][n]
+        assert alg[n] <= ceiling, f"{cfg} {n}: the restatement moved to {alg[n]:.3e} from fp32 eager"
         a, b = got[n].float().cpu(), ref_f32[n].float().cpu()
-        bound = FULL_TOL[cfg] + alg[n] + half_ulp(torch.maximum(a.abs(), b.abs()), got[n].dtype)
+        bound = FULL_TOL[cfg] + ceiling + half_ulp(torch.maximum(a.abs(), b.abs()), got[n].dtype)
         assert bool(((a - b).abs() <= bound).all()), f"{cfg} {n}: max-abs {e_f32[n]:.3e} vs fp32 eager"
     print(f"{cfg}: vs the backward from the saved output {e_model} | that restatement vs eager-fp32 {alg} | "
           f"reduced gradients vs eager-fp32 { {n: e_f32[n] for n in ('dBias', 'dMask')} } | eager-bf16's own { {n: e_self[n] for n in ('dBias', 'dMask')} }")

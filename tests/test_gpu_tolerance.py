@@ -74,6 +74,37 @@ def max_abs(a, b):
     return (a.float() - b.float()).abs().max().item()
 
 
+# What the two roundings the reference's kernels share with these (delta from the saved 16-bit output,
+# evoformer.py:313-323; the scaled query operand rounded once from head dim 32 on, :49, :433) cost dBias
+# against fp32 eager, measured with the oracle's restatement on one MI355X (C2 1.812e-2, C3 4.446e-2,
+# C4 4.153e-2, C5 2.651e-2) times 1.25.  Constants, so that the allowance cannot grow with a regression of
+# the forward's output; the measured values are printed.
+DBIAS_ROUNDINGS_CEILING = {"C2": 2.27e-2, "C3": 5.56e-2, "C4": 5.19e-2, "C5": 3.31e-2}
+_DBIAS_CACHE = {}
+
+
+def _dbias_fp32_distances(E, cfg):
+    """dBias written in fp32 at full size: its distance from fp32 eager, from the restatement with the two shared
+    roundings, and that restatement's own distance from fp32 eager (computed once per configuration)."""
+    if cfg not in _DBIAS_CACHE:
+        x = eager.make_inputs(cfg)
+        D = x["shape"][-1]
+        ref = eager_fp32_on_gpu(x)
+        got, kernels = c_abi_fwd_bwd(E, x, dbias_fp32=True)
+        xs = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in x.items()}
+        model = eager.backward_from_saved_output(xs["Q"], xs["K"], xs["V"], xs["mask"], xs["bias"], xs["dO"], got["O"], s_chunk=32,
+                                                 scaled_q_dtype=torch.bfloat16 if D > 16 else None)["dBias"]
+        saved_o = eager.backward_from_saved_output(xs["Q"], xs["K"], xs["V"], xs["mask"], xs["bias"], xs["dO"], got["O"], s_chunk=32)["dBias"]
+        d = {"err": max_abs(got["dBias"], ref["dBias"]), "own": max_abs(got["dBias"], model),
+             "cost_o": max_abs(saved_o, ref["dBias"]), "cost_oq": max_abs(model, ref["dBias"]),
+             "finite": bool(torch.isfinite(got["dBias"]).all()), "kernels": kernels, "mag": ref["dBias"].abs().max().item()}
+        print(f"\n{cfg} [{kernels}]: dBias (fp32 out) max-abs vs eager fp32 {d['err']:.3e} | vs the restatement with the saved output "
+              f"and the rounded scaled Q {d['own']:.3e} | restatement vs eager fp32: saved output alone {d['cost_o']:.3e}, both {d['cost_oq']:.3e} | "
+              f"max|dBias| {d['mag']:.2f}")
+        _DBIAS_CACHE[cfg] = d
+    return _DBIAS_CACHE[cfg]
+
+
 @pytest.mark.parametrize("cfg", ["C2", "C3", "C4", "C5"])
 def test_dbias_in_fp32_meets_the_stated_bound_at_full_size(E, cfg):
     """bf16 inputs and bf16 pair bias, dBias written in fp32, so no output rounding.
@@ -85,23 +116,29 @@ def test_dbias_in_fp32_meets_the_stated_bound_at_full_size(E, cfg):
            reference scales Q in Q's dtype (evoformer.py:49, 433): restated likewise (below head
            dim 32 the kernels carry the rounding residue and the scores are exact);
       (iii) the kernels' own arithmetic: held to a plain 2e-2 against the restatement with (i) and (ii).
-    Against fp32 eager itself the bound is 2e-2 plus what (i) and (ii) cost the restatement."""
-    x = eager.make_inputs(cfg)
-    D = x["shape"][-1]
-    ref = eager_fp32_on_gpu(x)
-    got, kernels = c_abi_fwd_bwd(E, x, dbias_fp32=True)
-    xs = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in x.items()}
-    model = eager.backward_from_saved_output(xs["Q"], xs["K"], xs["V"], xs["mask"], xs["bias"], xs["dO"], got["O"], s_chunk=32,
-                                             scaled_q_dtype=torch.bfloat16 if D > 16 else None)["dBias"]
-    saved_o = eager.backward_from_saved_output(xs["Q"], xs["K"], xs["V"], xs["mask"], xs["bias"], xs["dO"], got["O"], s_chunk=32)["dBias"]
-    err, own = max_abs(got["dBias"], ref["dBias"]), max_abs(got["dBias"], model)
-    cost_o, cost_oq = max_abs(saved_o, ref["dBias"]), max_abs(model, ref["dBias"])
-    print(f"\n{cfg} [{kernels}]: dBias (fp32 out) max-abs vs eager fp32 {err:.3e} | vs the restatement with the saved output "
-          f"and the rounded scaled Q {own:.3e} | restatement vs eager fp32: saved output alone {cost_o:.3e}, both {cost_oq:.3e} | "
-          f"max|dBias| {ref['dBias'].abs().max().item():.2f}")
-    assert torch.isfinite(got["dBias"]).all()
-    assert own <= TOL, f"{cfg}: dBias max-abs {own:.3e} > {TOL} against the restatement"
-    assert err <= TOL + cost_oq, f"{cfg}: dBias max-abs {err:.3e} vs fp32 eager"
+    Against fp32 eager itself the bound is 2e-2 plus a constant ceiling per configuration on what (i) and
+    (ii) cost; the restatement's own distance is held under that ceiling too, so neither can drift."""
+    d = _dbias_fp32_distances(E, cfg)
+    assert d["finite"]
+    assert d["own"] <= TOL, f"{cfg}: dBias max-abs {d['own']:.3e} > {TOL} against the restatement"
+    assert d["cost_oq"] <= DBIAS_ROUNDINGS_CEILING[cfg], f"{cfg}: the restatement moved to {d['cost_oq']:.3e} from fp32 eager"
+    assert d["err"] <= TOL + DBIAS_ROUNDINGS_CEILING[cfg], f"{cfg}: dBias max-abs {d['err']:.3e} vs fp32 eager"
+
+
+_SHARED_ROUNDINGS = ("delta from the saved bf16 output (evoformer.py:313-323) and, at head dim 32, the scaled query operand "
+                     "rounded once (evoformer.py:49, 433) put fp32-written dBias beyond a plain 2e-2 of fp32 eager here "
+                     "(4.4e-2, 4.2e-2, 2.7e-2 measured): the stated bound is not met on this configuration")
+
+
+@pytest.mark.parametrize("cfg", ["C2",
+                                 pytest.param("C3", marks=pytest.mark.xfail(strict=True, reason=_SHARED_ROUNDINGS)),
+                                 pytest.param("C4", marks=pytest.mark.xfail(strict=True, reason=_SHARED_ROUNDINGS)),
+                                 pytest.param("C5", marks=pytest.mark.xfail(strict=True, reason=_SHARED_ROUNDINGS))])
+def test_dbias_in_fp32_within_a_plain_2e_2_of_fp32_eager(E, cfg):
+    """The bound as stated, with nothing added: fp32-written dBias within 2e-2 max-abs of fp32 eager.  Holds at C2
+    (1.9e-2); the other three configurations are expected failures, kept so that the gap stays visible."""
+    d = _dbias_fp32_distances(E, cfg)
+    assert d["err"] <= TOL, f"{cfg}: dBias max-abs {d['err']:.3e} vs fp32 eager"
 
 
 def test_c5_shape_in_fp16_meets_the_stated_bound(E):
