@@ -35,7 +35,10 @@ static int check_common(const EvoAttnParams *p) {
     if (p->mask_kind < EVO_MASK_NONE || p->mask_kind > EVO_MASK_F16) return EVO_EINVAL;
     if ((p->bias_dtype == EVO_NONE) != (p->bias == nullptr)) return EVO_EINVAL;
     if ((p->mask_kind == EVO_MASK_NONE) != (p->mask == nullptr)) return EVO_EINVAL;
-    if (!p->q || !p->k || !p->v || !p->o || !p->lse) return EVO_EINVAL;
+    if (!p->q || !p->k || !p->v || !p->lse) return EVO_EINVAL;
+    // (with a gate the gated output may stand alone: the forward then writes no ungated O and the backward,
+    // whose gate pass forms delta from the gated output, reads none)
+    if (!p->o && !(p->gate && p->o_gated)) return EVO_EINVAL;
     if (!(p->scale == p->scale) || p->scale <= 0.0f) return EVO_EINVAL;
     if (p->flags & ~EVO_FLAG_ALL) return EVO_EINVAL;
     // (a second call on the same dout would apply the gate to it a second time)
@@ -301,7 +304,7 @@ static int check_bwd(const EvoAttnParams *p) {
         if (!aligned(p->dbias, elem_size(p->dbias_dtype))) return EVO_EALIGN;
     }
     if (p->dmask && !aligned(p->dmask, 4)) return EVO_EALIGN;
-    if (p->gate && (!p->dgate || !aligned(p->dgate, 16) || !aligned(p->dout, 16) || !aligned(p->o, 16))) return p->dgate ? EVO_EALIGN : EVO_EINVAL;
+    if (p->gate && (!p->dgate || !aligned(p->dgate, 16) || !aligned(p->dout, 16) || !aligned(p->o, 16) || !aligned(p->o_gated, 16))) return p->dgate ? EVO_EALIGN : EVO_EINVAL;
     const WsLayout w = ws_layout(*p);
     if (!p->workspace || p->workspace_bytes < w.total) return EVO_EWORKSPACE;
     if (!aligned(p->workspace, 256)) return EVO_EALIGN;
@@ -465,9 +468,10 @@ int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
     if (p0->gate) {
         // (in place: a thread reads its 8 elements of dout before it writes them)
         void *d_o = (p0->flags & EVO_FLAG_GATE_DOUT_INPLACE) ? const_cast<void *>(p0->dout) : (void *)(ws + w.dout_ungated);
-        if ((rc = launch_gate_bwd(*p0, d_o, st))) return rc;
+        if ((rc = launch_gate_bwd(*p0, d_o, (float *)(ws + w.delta), st))) return rc;
         ungated.dout = d_o;
         ungated.gate = nullptr;
+        ungated.o_gated = nullptr;
     }
     const EvoAttnParams *p = &ungated;
     Extra e{};
@@ -475,6 +479,7 @@ int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
     e.chunk = w.chunk;
     e.vec_ok = bias_vec_ok(*p);
     e.delta = (float *)(ws + w.delta);
+    e.delta_given = p0->gate ? 1 : 0;   // (the gate's pass wrote it; the dQ kernels then read no ungated O)
     e.shift = (float *)(ws + w.shift);
     e.dmask_part = (float *)(ws + w.dmask_part);
     e.dbias_part = (float *)(ws + w.dbias_part);

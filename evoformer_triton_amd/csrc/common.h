@@ -38,6 +38,7 @@ struct Extra {
     int bias_batches;  // 1 when one bias is shared by the whole batch, else B
     int bias_direct;   // the one-workgroup-per-problem kernels read the bias from the caller's tensor, not from bq / bk
     int dbias_chunks;  // > 0: the dK/dV kernel over a chunk of rows also sums that many dBias partials (else `dbias_reduce` does)
+    int delta_given;   // `delta` already holds rowsum(dO * O) (the gate's pass wrote it): the dQ kernels read it and do not touch o
     float *delta;      // [B][H][S][N]
     float *shift;      // [B][S] per-row mask shift (plain kernels)
     float *dbias_part; // [n_chunks][B][H][N][N]

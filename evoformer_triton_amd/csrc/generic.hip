@@ -59,9 +59,11 @@ __global__ void __launch_bounds__(64) gen_fwd(EvoAttnParams p) {
         m = mn;
     }
     if (row < p.N) {
-        T *O = (T *)p.o + pr.base + (int64_t)row * p.stride_n;
         float inv = 1.0f / l;
-        for (int d = 0; d < D; ++d) O[d] = (T)(acc[d] * inv);
+        if (p.o) {   // (with a gate the caller may ask for the gated output alone)
+            T *O = (T *)p.o + pr.base + (int64_t)row * p.stride_n;
+            for (int d = 0; d < D; ++d) O[d] = (T)(acc[d] * inv);
+        }
         if (p.gate) {
             const int64_t off = pr.base + (int64_t)row * p.stride_n;
             const T *Gt = (const T *)p.gate + off;
@@ -326,20 +328,24 @@ int launch_delta_generic(const EvoAttnParams &p, const Extra &e, hipStream_t st)
     return EVO_OK;
 }
 
-// The gate's own backward, one pass over the rows: from the gradient of sigmoid(g) * O (in
-// p.dout), the gate logits g and the ungated O,
-//     dO = dout * sigmoid(g)                        -> dout_ungated (what the attention backward runs on)
-//     dg = dout * O * sigmoid(g) * (1 - sigmoid(g)) -> p.dgate
-// all three laid out like q.  One thread per 8 consecutive head-dim elements of one row.
-template <typename T>
-__global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_ungated) {
-    const int cpr = p.D / 8;   // 8-element pieces per row
+// The gate's own backward, one pass over the rows: from the gradient of Og = sigmoid(g) * O (in
+// p.dout), the gate logits g and the forward's output, gated (p.o_gated) or, where that is not
+// given, ungated (p.o),
+//     dO    = dout * sigmoid(g)                           -> dout_ungated (what the attention backward runs on)
+//     dg    = dout * Og * (1 - sigmoid(g))                -> p.dgate       (= dout * O * sigmoid(g) * (1 - sigmoid(g)))
+//     delta = sum over the head dim of dout * Og          -> delta         (= rowsum(dO * O), from unrounded products)
+// the first two laid out like q, delta [B][H][S][N].  With delta formed here the dQ kernels need no
+// ungated O, so the forward need not write one.  One thread per 8 consecutive head-dim elements of
+// one row; the D / 8 threads of a row are neighbours in a wave and add their parts of delta.
+template <typename T, bool FROM_GATED>
+__global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_ungated, float *delta) {
+    const int cpr = p.D / 8;   // 8-element pieces per row (1, 2, 4, 8 or 16)
     const int64_t pieces = (int64_t)p.B * p.H * p.S * p.N * cpr;
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= pieces) return;
+    const int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t i = i0 < pieces ? i0 : pieces - 1;   // (the threads past the end keep the row sums below whole)
     const int c = (int)(i % cpr);
     const int64_t r = i / cpr;
-    int64_t off;
+    int64_t off, drow;
     if (p.stride_h < p.stride_n) {
         // heads inside a token (the per-head layout): rows in the order they lie in memory, (b, s, n, h), so that
         // a wave's pieces are neighbours (in problem order they are one head's 16 D bytes out of every token)
@@ -348,16 +354,20 @@ __global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_
         const int n = (int)(tok % p.N);
         const int64_t bs = tok / p.N;
         off = (bs / p.S) * p.stride_b + (bs % p.S) * p.stride_s + (int64_t)n * p.stride_n + (int64_t)h * p.stride_h + c * 8;
+        drow = (((bs / p.S) * p.H + h) * p.S + bs % p.S) * p.N + n;
     } else {
         const Prob pr = decode_problem(p, (unsigned)(r / p.N));
         off = pr.base + (r % p.N) * p.stride_n + c * 8;
+        drow = r;
     }
-    const T *go = (const T *)p.dout + off, *gl = (const T *)p.gate + off, *o = (const T *)p.o + off;
+    const T *go = (const T *)p.dout + off, *gl = (const T *)p.gate + off;
+    const T *o = (const T *)(FROM_GATED ? p.o_gated : p.o) + off;
     T *d_o = dout_ungated + off, *d_g = (T *)p.dgate + off;
     // eight elements at a time: 16-byte loads and stores for the 16-bit types (the pieces are
     // 16-byte aligned: dense tensors, head dim a multiple of 8), two of each for fp32
     constexpr int V = sizeof(T) == 2 ? 8 : 4;
     typedef T vec __attribute__((ext_vector_type(V)));
+    float dsum = 0.0f;
 #pragma unroll
     for (int j0 = 0; j0 < 8; j0 += V) {
         const vec a = *reinterpret_cast<const vec *>(go + j0), b = *reinterpret_cast<const vec *>(gl + j0),
@@ -367,20 +377,34 @@ __global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_
         for (int j = 0; j < V; ++j) {
             const float sg = 1.0f / (1.0f + expf(-(float)b[j]));
             const float gr = (float)a[j];
+            const float og = FROM_GATED ? (float)c2[j] : (float)c2[j] * sg;   // sigmoid(g) * O
             r_o[j] = (T)(gr * sg);
-            r_g[j] = (T)(gr * (float)c2[j] * sg * (1.0f - sg));
+            r_g[j] = (T)(gr * og * (1.0f - sg));
+            dsum = fmaf(gr, og, dsum);
         }
-        *reinterpret_cast<vec *>(d_o + j0) = r_o;
-        *reinterpret_cast<vec *>(d_g + j0) = r_g;
+        if (i0 < pieces) {
+            *reinterpret_cast<vec *>(d_o + j0) = r_o;
+            *reinterpret_cast<vec *>(d_g + j0) = r_g;
+        }
     }
+    for (int w = 1; w < cpr; w <<= 1) dsum += __shfl_xor(dsum, w);
+    if (c == 0 && i0 < pieces) delta[drow] = dsum;
 }
 
-int launch_gate_bwd(const EvoAttnParams &p, void *dout_ungated, hipStream_t st) {
+int launch_gate_bwd(const EvoAttnParams &p, void *dout_ungated, float *delta, hipStream_t st) {
     const int64_t pieces = (int64_t)p.B * p.H * p.S * p.N * (p.D / 8);
     const unsigned grid = (unsigned)((pieces + 255) / 256);
-    if (p.dtype == EVO_F32) gate_bwd_kernel<float><<<grid, 256, 0, st>>>(p, (float *)dout_ungated);
-    else if (p.dtype == EVO_BF16) gate_bwd_kernel<bf16_t><<<grid, 256, 0, st>>>(p, (bf16_t *)dout_ungated);
-    else gate_bwd_kernel<f16_t><<<grid, 256, 0, st>>>(p, (f16_t *)dout_ungated);
+    const bool g = p.o_gated != nullptr;
+    if (p.dtype == EVO_F32) {
+        if (g) gate_bwd_kernel<float, true><<<grid, 256, 0, st>>>(p, (float *)dout_ungated, delta);
+        else gate_bwd_kernel<float, false><<<grid, 256, 0, st>>>(p, (float *)dout_ungated, delta);
+    } else if (p.dtype == EVO_BF16) {
+        if (g) gate_bwd_kernel<bf16_t, true><<<grid, 256, 0, st>>>(p, (bf16_t *)dout_ungated, delta);
+        else gate_bwd_kernel<bf16_t, false><<<grid, 256, 0, st>>>(p, (bf16_t *)dout_ungated, delta);
+    } else {
+        if (g) gate_bwd_kernel<f16_t, true><<<grid, 256, 0, st>>>(p, (f16_t *)dout_ungated, delta);
+        else gate_bwd_kernel<f16_t, false><<<grid, 256, 0, st>>>(p, (f16_t *)dout_ungated, delta);
+    }
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }
@@ -406,7 +430,7 @@ int launch_mask_shift(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 }
 
 int launch_generic_bwd(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
-    int rc = launch_delta_generic(p, e, st);
+    int rc = e.delta_given ? EVO_OK : launch_delta_generic(p, e, st);
     if (rc) return rc;
     rc = launch_mask_shift(p, e, st);
     if (rc) return rc;

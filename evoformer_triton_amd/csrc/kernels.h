@@ -11,7 +11,7 @@ int launch_generic_bwd(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_delta_generic(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_dmask_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 int launch_dbias_reduce(const EvoAttnParams &p, const Extra &e, hipStream_t st);
-int launch_gate_bwd(const EvoAttnParams &p, void *dout_ungated, hipStream_t st);  // dO and dgate from the gradient of the gated output
+int launch_gate_bwd(const EvoAttnParams &p, void *dout_ungated, float *delta, hipStream_t st);  // dO, dgate and delta from the gradient of the gated output
 int launch_mask_shift(const EvoAttnParams &p, const Extra &e, hipStream_t st);
 
 int launch_prep(const EvoAttnParams &p, const Extra &e, hipStream_t st);

@@ -126,7 +126,9 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
         const unsigned pid = (bh * (unsigned)p.S) + s;
         const Prob pr = decode_problem(p, pid);
         const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
-        const T *Gd = (const T *)p.dout + pr.base, *O = (const T *)p.o + pr.base;
+        const T *Gd = (const T *)p.dout + pr.base;
+        // (where delta is given, by the gate's pass, there may be no ungated O: the loads go to dO instead and their sum is dropped)
+        const T *O = e.delta_given ? Gd : (const T *)p.o + pr.base;
         const uint2 *m2row = e.m2 + ((int64_t)b * p.S + s) * npad;
         const bool dead = e.dead[b * p.S + s] != 0;
         const bool kill = dead && p.mask_kind == EVO_MASK_BOOL;
@@ -149,9 +151,9 @@ __global__ void __launch_bounds__(256) mfma_dq(EvoAttnParams p, Extra e) {
                 dpart = dot8<T>(gf[ks], oraw, dpart);
             }
         }
-        const float dl = dpart + __shfl_xor(dpart, 32);
+        const float dl = e.delta_given ? e.delta[pr.row0 + qrow] : dpart + __shfl_xor(dpart, 32);
         const float lse2 = p.lse[pr.row0 + qrow] * kLog2e;
-        if (wave == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
+        if (!e.delta_given && wave == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             if (ks * 16 + g * 8 == AUGC) {

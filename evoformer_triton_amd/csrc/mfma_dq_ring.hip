@@ -61,7 +61,8 @@ struct RingGeo {
     static constexpr int OFF_G = OFF_Q + Q_BYTES;
     static constexpr int OFF_O = OFF_G + Q_BYTES;
     static constexpr int OFF_L = OFF_O + Q_BYTES;                   // -log2-sum-exp of the QR query rows as (hi, mid, lo, 0)
-    static constexpr int STAGE_BYTES = OFF_L + QR * 8;
+    static constexpr int OFF_DL = OFF_L + QR * 8;                   // delta of the QR query rows (fp32), where it is given
+    static constexpr int STAGE_BYTES = OFF_DL + QR * 4;
     static constexpr int RED_BYTES = 8 * 32 * RP * 4;
     static constexpr int STAGE_1K = (STAGE_BYTES + 1023) / 1024 * 1024;
     // The partial dQ tiles get LDS of their own where 160 KB allow it; otherwise they lie in the
@@ -175,6 +176,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     struct Staged {
         u32x4 v[IPW];
         float lse;
+        float dl;   // delta, where it is given
     };
     // element offset of row 0 of problem (b, h, s_begin); S row s is (s - s_begin) * stride_s on
     const int64_t base0 = (int64_t)b * p.stride_b + (int64_t)h * p.stride_h + (int64_t)s_begin * p.stride_s;
@@ -202,7 +204,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             else if (n < 2 * R::I_K) { base = (const T *)p.v; m = n - R::I_K; row0 = blk * BKV; off = R::OFF_V; }
             else if (n < R::I_KVA + R::I_Q) { base = (const T *)p.q; m = n - R::I_KVA; row0 = qbase; off = R::OFF_Q; }
             else if (n < R::I_KVA + 2 * R::I_Q) { base = (const T *)p.dout; m = n - R::I_KVA - R::I_Q; row0 = qbase; off = R::OFF_G; }
-            else { base = (const T *)p.o; m = n - R::I_KVA - 2 * R::I_Q; row0 = qbase; off = R::OFF_O; }
+            else {   // (where delta is given there may be no ungated O: the piece is dO once more, and is not used)
+                base = e.delta_given ? (const T *)p.dout : (const T *)p.o; m = n - R::I_KVA - 2 * R::I_Q; row0 = qbase; off = R::OFF_O;
+            }
             const int L = m * 64 + lane;
             const int r = L / C, cpos = L % C;
             const int ch = cpos ^ ((r / R::RPB) % C);
@@ -259,8 +263,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         // wave asks, wave 0 stores): a load whose result is carried into the next row's
         // prologue in a register would make that prologue wait for everything requested here
         if (i1 >= IPW) {
-            if (NBLK == 1) stg.lse = flse[flse_off];
-            else stg.lse = p.lse[((int64_t)bh * p.S + s_begin + row) * p.N + min(qbase + lane, p.N - 1)];
+            const int64_t lrow = NBLK == 1 ? 0 : ((int64_t)bh * p.S + s_begin + row) * p.N;
+            const float *lsrc = NBLK == 1 ? flse : p.lse + lrow;
+            stg.lse = lsrc[flse_off];
+            // (delta has the layout of the log-sum-exp: the same offset from its own base)
+            if (e.delta_given) stg.dl = (e.delta + (lsrc - p.lse))[flse_off];
         }
     };
     auto fetch = [&](Staged &stg, int t) { fetch_part(stg, t, 0, IPW); };
@@ -290,8 +297,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg.v[i];
             }
         }
-        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR)
+        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR) {
             *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-stg.lse * kLog2e);
+            if (e.delta_given) *reinterpret_cast<float *>(buf + R::OFF_DL + lane * 4) = stg.dl;
+        }
     };
     auto stash = [&](const Staged &stg, int t, int par) { stash_part(stg, t, 0, IPW, par); };
 
@@ -433,7 +442,8 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
                     dl = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
                 }
-                if (kq == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
+                if (e.delta_given) dl = *reinterpret_cast<const float *>(buf + R::OFF_DL + (qi * 32 + li) * 4);   // uniform
+                else if (kq == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     if (ks * 16 + g * 8 == AUGC) {

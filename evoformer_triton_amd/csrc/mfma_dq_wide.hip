@@ -63,7 +63,9 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
     const int q0 = (lid % nqb) * BQ + wave * 32;
     const Prob pr = walk_problem(p, pid);
     const T *Q = (const T *)p.q + pr.base, *K = (const T *)p.k + pr.base, *V = (const T *)p.v + pr.base;
-    const T *Gd = (const T *)p.dout + pr.base, *O = (const T *)p.o + pr.base;
+    const T *Gd = (const T *)p.dout + pr.base;
+    // (where delta is given, by the gate's pass, there may be no ungated O: the loads go to dO instead and their sum is dropped)
+    const T *O = e.delta_given ? Gd : (const T *)p.o + pr.base;
     const int64_t sn = p.stride_n;
     const bool active = q0 < p.N;   // wave-uniform
     const int qrow = min(q0 + li, p.N - 1);
@@ -126,9 +128,9 @@ __global__ void __launch_bounds__(NW * 64, D >= 128 ? 1 : NW == 8 ? (D <= 32 ? 4
             dpart = dot8<T>(gf[ks], oraw, dpart);
         }
     }
-    const float dl = dpart + __shfl_xor(dpart, 32);
+    const float dl = e.delta_given ? e.delta[pr.row0 + qrow] : dpart + __shfl_xor(dpart, 32);
     const float lse2 = p.lse[pr.row0 + qrow] * kLog2e;
-    if (g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
+    if (!e.delta_given && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
         if (ks * 16 + g * 8 == AUGC) {

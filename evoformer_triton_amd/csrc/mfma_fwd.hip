@@ -354,15 +354,17 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
             T *O = (T *)p.o + pr.base + (int64_t)q * sn;
             // natural-log LSE of the (shifted) scores, as the reference stores it (:285-288)
             if (g == 0) p.lse[pr.row0 + q] = (m + __log2f(l)) * kLn2;
+            if (p.o) {   // uniform (with a gate the caller may ask for the gated output alone)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int d0 = dt * 32 + 8 * rr + 4 * g;
-                    if (d0 < D)
-                        store4<T>(O + d0, oacc[dt][4 * rr] * inv, oacc[dt][4 * rr + 1] * inv,
-                                  oacc[dt][4 * rr + 2] * inv, oacc[dt][4 * rr + 3] * inv);
-                }
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int d0 = dt * 32 + 8 * rr + 4 * g;
+                        if (d0 < D)
+                            store4<T>(O + d0, oacc[dt][4 * rr] * inv, oacc[dt][4 * rr + 1] * inv,
+                                      oacc[dt][4 * rr + 2] * inv, oacc[dt][4 * rr + 3] * inv);
+                    }
+            }
             if (p.gate) {   // uniform: sigmoid(gate) * O goes out as a second tensor, from the same registers
                 const int64_t off = pr.base + (int64_t)q * sn;
                 T *Og = (T *)p.o_gated + off;

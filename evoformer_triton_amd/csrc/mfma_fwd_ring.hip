@@ -548,8 +548,10 @@ __global__ void __launch_bounds__(512) mfma_fwd_ring(EvoAttnParams p, Extra e) {
             if (q < p.N) {
                 T *O = (T *)p.o + base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
                 if (g == 0) p.lse[(int64_t)pid * p.N + q] = (m + __log2f(l)) * kLn2;
+                if (!GATED || p.o) {   // uniform (with a gate the caller may ask for the gated output alone)
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) store_row_tile<T>(O, dt * 32, D, oacc[dt], inv, g);
+                    for (int dt = 0; dt < DT; ++dt) store_row_tile<T>(O, dt * 32, D, oacc[dt], inv, g);
+                }
                 if constexpr (GATED) {   // sigmoid(gate) * O goes out as a second tensor, from the same registers
                     const int64_t off = base0 + (int64_t)t * p.stride_s + (int64_t)q * sn;
 #pragma unroll

@@ -202,7 +202,8 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False, gate=None)
     mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
     bias, bias_dt, bstr = _prep_bias(pair_bias, B, H, N, Q.dtype, Q.device)
     with _on_device(Q.device):
-        O = torch.empty_like(Qp)                               # evoformer.py:654
+        # (with a gate only the gated output is written: the backward's gate pass forms delta from it)
+        O = None if gate is not None else torch.empty_like(Qp)  # evoformer.py:654
         lse = torch.empty((B, H, S, N), device=Q.device, dtype=torch.float32)   # :669-671
         p = _params(Qp, Kp, Vp, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
         nbytes = _prep_bytes_upper(lib, p) if prep_upper else lib.evoattn_prep_bytes(ctypes.byref(p))
@@ -215,10 +216,10 @@ def _fwd_impl(Q, K, V, res_mask, pair_bias, layout, prep_upper=False, gate=None)
             p.gate, p.o_gated = _ptr(Gp), _ptr(Og)
         _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(Q.device)), "evoattn_fwd")
         if Dp != D:
-            O = O[..., :D].contiguous()
+            O = None if O is None else O[..., :D].contiguous()
             Og = None if Og is None else Og[..., :D].contiguous()
-    if gate is not None:
-        return Qc, Kc, Vc, mask, bias, O, lse, prep, (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype)), \
+    if gate is not None:   # (the gated output stands where the ungated one does: it is what the backward is given)
+        return Qc, Kc, Vc, mask, bias, Og, lse, prep, (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype)), \
             (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype)), Og
     mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
@@ -242,8 +243,9 @@ def _forward(ctx, Q, K, V, res_mask, pair_bias, layout):
 def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_meta, need_dmask, need_dbias,
               prep_valid=True, gate=None):
     """Allocate the gradients and the workspace and enqueue the backward; `mask` and `bias`
-    are the tensors the forward's kernels saw.  Returns (dQ, dK, dV, dmask, dbias) with the
-    last two in the shape and dtype of the caller's tensors, or None."""
+    are the tensors the forward's kernels saw.  With `gate`, `O` is the gated output sigmoid(gate) * O
+    and dO its gradient.  Returns (dQ, dK, dV, dmask, dbias) with the last two in the shape and dtype
+    of the caller's tensors, or None."""
     lib = _lib.load()
     B, S, N, H, D = Q.shape
     mask_kind, mstr, mask_orig = mask_meta
@@ -266,7 +268,7 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
     want_dmask = bool(need_dmask and mask is not None and mask.is_floating_point())
     with _on_device(Q.device):
         dQ, dK, dV = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)   # :749-751
-        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, O, lse, layout, head_dim=D)
+        p = _params(Q, K, V, mask, mask_kind, mstr, bias, bias_dt, bstr, None if gate is not None else O, lse, layout, head_dim=D)
         p.dout, p.dq, p.dk, p.dv = _ptr(dO), _ptr(dQ), _ptr(dK), _ptr(dV)
         dbias = dmask = None
         if want_dbias:
@@ -279,7 +281,7 @@ def _bwd_impl(dO, Q, K, V, mask, bias, O, lse, prep, layout, mask_meta, bias_met
         dgate = None
         if gate is not None:                                     # dO here is the gradient of the gated output
             dgate = torch.empty_like(Q)
-            p.gate, p.dgate = _ptr(gate), _ptr(dgate)
+            p.gate, p.dgate, p.o_gated = _ptr(gate), _ptr(dgate), _ptr(O)
         ws = _alloc_bytes(lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)), Q.device)
         p.workspace, p.workspace_bytes = _ptr(ws), ws.numel()
         if not prep_valid:                                       # not the forward's tensors: prepare again
@@ -409,25 +411,25 @@ _op_fwd.register_autograd(_op_backward, setup_context=_op_setup_context)
 @torch.library.custom_op("evoattn::fwd_gated", mutates_args=(), device_types="cuda")
 def _op_fwd_gated(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
                   pair_bias: Optional[torch.Tensor], gate: torch.Tensor, per_head: bool
-                  ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(O_gated, O, LSE, prep bytes, seen): `evoattn::fwd` with the output gate applied in the epilogue;
-    the ungated O is returned as well because the backward takes delta from it."""
+                  ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(O_gated, LSE, prep bytes, seen): `evoattn::fwd` with the output gate applied in the epilogue.  No
+    ungated O is written: the backward takes delta and the gate's gradient from the gated output."""
     out = _fwd_impl(Q, K, V, res_mask, pair_bias, "ds4sci" if per_head else "reference", prep_upper=True, gate=gate)
-    return out[10], out[5], out[6], out[7], _seen(out[3], out[4])
+    return out[10], out[6], out[7], _seen(out[3], out[4])
 
 
 @_op_fwd_gated.register_fake
 def _(Q, K, V, res_mask, pair_bias, gate, per_head):
     o, lse, prep, seen = torch.ops.evoattn.fwd(Q, K, V, res_mask, pair_bias, per_head)
-    return Q.new_empty(Q.shape), o, lse, prep, seen
+    return o, lse, prep, seen
 
 
 @torch.library.custom_op("evoattn::bwd_gated", mutates_args=(), device_types="cuda")
 def _op_bwd_gated(dOg: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, res_mask: Optional[torch.Tensor],
-                  pair_bias: Optional[torch.Tensor], gate: torch.Tensor, O: torch.Tensor, lse: torch.Tensor,
+                  pair_bias: Optional[torch.Tensor], gate: torch.Tensor, Og: torch.Tensor, lse: torch.Tensor,
                   prep: torch.Tensor, seen: torch.Tensor, per_head: bool, need_dbias: bool, need_dmask: bool
                   ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(dQ, dK, dV, dMask, dBias, dGate) from the gradient of the gated output."""
+    """(dQ, dK, dV, dMask, dBias, dGate) from the gradient of the gated output Og and Og itself."""
     B, S, N, H, D = Q.shape
     Qc, Kc, Vc = Q.contiguous(), K.contiguous(), V.contiguous()
     mask, mask_kind, mstr = _prep_mask(res_mask, B, S, N, Q.device)
@@ -435,7 +437,7 @@ def _op_bwd_gated(dOg: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.
     mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
     bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
     same = bool(torch.equal(seen.cpu(), _seen(mask, bias)))
-    dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Qc, Kc, Vc, mask, bias, O.contiguous(), lse, prep,
+    dQ, dK, dV, dmask, dbias, dgate = _bwd_impl(dOg, Qc, Kc, Vc, mask, bias, Og.contiguous(), lse, prep,
                                                 "ds4sci" if per_head else "reference", mask_meta, bias_meta,
                                                 need_dmask, need_dbias, prep_valid=same, gate=_check_gate(gate, Qc))
     none = Q.new_empty((0,))
@@ -443,7 +445,7 @@ def _op_bwd_gated(dOg: torch.Tensor, Q: torch.Tensor, K: torch.Tensor, V: torch.
 
 
 @_op_bwd_gated.register_fake
-def _(dOg, Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen, per_head, need_dbias, need_dmask):
+def _(dOg, Q, K, V, res_mask, pair_bias, gate, Og, lse, prep, seen, per_head, need_dbias, need_dmask):
     want_dmask = need_dmask and res_mask is not None and res_mask.is_floating_point()
     want_dbias = need_dbias and pair_bias is not None
     return (Q.new_empty(Q.shape), Q.new_empty(Q.shape), Q.new_empty(Q.shape),
@@ -453,12 +455,12 @@ def _(dOg, Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen, per_head, nee
 
 def _op_gated_setup_context(ctx, inputs, output):
     Q, K, V, res_mask, pair_bias, gate, per_head = inputs
-    Og, O, lse, prep, seen = output
-    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen)
+    Og, lse, prep, seen = output
+    ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, Og, lse, prep, seen)
     ctx.per_head = per_head
 
 
-def _op_gated_backward(ctx, dOg, dO_unused, dlse, dprep, dseen):
+def _op_gated_backward(ctx, dOg, dlse, dprep, dseen):
     Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen = ctx.saved_tensors
     need_dmask = bool(ctx.needs_input_grad[3] and res_mask is not None and res_mask.is_floating_point())
     need_dbias = bool(ctx.needs_input_grad[4] and pair_bias is not None)
@@ -506,16 +508,16 @@ class _PerHeadAttention(torch.autograd.Function):
 class _GatedAttention(torch.autograd.Function):
     """sigmoid(gate) * attention(Q, K, V, res_mask, pair_bias) with the gate applied in the forward
     kernel's epilogue (the step that follows the attention in an Evoformer block; the reference
-    returns O ungated, evoformer.py:735).  `gate`: the gate logits, shaped like Q.  The ungated O is
-    kept for the backward, which returns the gate's gradient as a sixth value.  Under torch.compile the
+    returns O ungated, evoformer.py:735).  `gate`: the gate logits, shaped like Q.  No ungated O is written:
+    the gated output is kept for the backward, which returns the gate's gradient as a sixth value.  Under torch.compile the
     same work goes through torch.ops.evoattn.fwd_gated / .bwd_gated."""
 
     @staticmethod
     def forward(ctx, Q, K, V, res_mask, pair_bias, gate, layout):
         if torch.compiler.is_compiling():
             # under torch.compile the device work is the registered operator (opaque to the tracer)
-            Og, O, lse, prep, seen = torch.ops.evoattn.fwd_gated(Q, K, V, res_mask, pair_bias, gate, layout == "ds4sci")
-            ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, O, lse, prep, seen)
+            Og, lse, prep, seen = torch.ops.evoattn.fwd_gated(Q, K, V, res_mask, pair_bias, gate, layout == "ds4sci")
+            ctx.save_for_backward(Q, K, V, res_mask, pair_bias, gate, Og, lse, prep, seen)
             ctx.layout, ctx.through_ops = layout, True
             return Og
         Qc, Kc, Vc, mask, bias, O, lse, prep, mask_meta, bias_meta, Og = _fwd_impl(Q, K, V, res_mask, pair_bias, layout,
@@ -565,8 +567,8 @@ class _SlotAttention(torch.autograd.Function):
     slots by their strides (a token's row lies W*H*D elements from the next); nothing is copied.  Every
     tensor the kernels lay out like Q is a slot of a buffer of that shape:
 
-        outputs OB   slot 0  O (ungated, kept for the backward)     gradients DP   slot 0  dQ
-                     slot 1  sigmoid(g) * O (returned when gated)                  slot 1  dK
+        outputs OB   slot 0  O (without a gate; kept for the backward) gradients DP   slot 0  dQ
+                     slot 1  sigmoid(g) * O (with a gate; likewise)               slot 1  dK
                      slot 2  the gradient coming back (dO)                         slot 2  dV
                      slot 3  -                                                     slot 3  dgate
 
@@ -589,7 +591,8 @@ class _SlotAttention(torch.autograd.Function):
             p = _SlotAttention._params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
             prep = _alloc_bytes(lib.evoattn_prep_bytes(ctypes.byref(p)), P.device)
             p.prep, p.prep_bytes = _ptr(prep), prep.numel()
-            if gated:
+            if gated:         # the gated output alone: slot 0 stays unwritten
+                p.o = None
                 p.gate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(OB[:, :, :, 1])
             _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(P.device)), "evoattn_fwd")
         ctx.save_for_backward(P, mask, bias, lse, prep)
@@ -635,7 +638,8 @@ class _SlotAttention(torch.autograd.Function):
             p = _SlotAttention._params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
             p.dout, p.dq, p.dk, p.dv = _ptr(slot), _ptr(DP[:, :, :, 0]), _ptr(DP[:, :, :, 1]), _ptr(DP[:, :, :, 2])
             if ctx.gated:     # slot 2 is this Function's own memory: the gradient of the ungated output takes its place
-                p.gate, p.dgate = _ptr(P[:, :, :, 3]), _ptr(DP[:, :, :, 3])
+                p.o = None    # (delta and the gate's gradient come from the gated output, slot 1)
+                p.gate, p.dgate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(DP[:, :, :, 3]), _ptr(OB[:, :, :, 1])
                 p.flags |= _lib.EVO_FLAG_GATE_DOUT_INPLACE
             dbias = dmask = None
             if want_dbias:

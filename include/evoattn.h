@@ -31,8 +31,9 @@
 extern "C" {
 #endif
 
-#define EVOATTN_VERSION 3   /* 2: gate, o_gated, dgate appended to EvoAttnParams; 3: LayerNorm and column-sum entry points,
-                               EVO_FLAG_GATE_DOUT_INPLACE, a gate on a q-family with gaps (slots of a wider buffer) */
+#define EVOATTN_VERSION 4   /* 2: gate, o_gated, dgate appended to EvoAttnParams; 3: LayerNorm and column-sum entry points,
+                               EVO_FLAG_GATE_DOUT_INPLACE, a gate on a q-family with gaps (slots of a wider buffer);
+                               4: with a gate `o` may be NULL (the gated output alone), the backward takes o_gated */
 
 /* element types */
 enum {
@@ -124,7 +125,7 @@ typedef struct EvoAttnParams {
     const void *q, *k, *v;
     const void *bias;     /* may be NULL (bias_dtype = EVO_NONE) */
     const void *mask;     /* may be NULL (mask_kind = EVO_MASK_NONE) */
-    void       *o;        /* fwd: out; bwd: in */
+    void       *o;        /* fwd: out; bwd: in (may be NULL with a gate, see below) */
     float      *lse;      /* fwd: out; bwd: in */
 
     const void *dout;     /* bwd only below */
@@ -143,14 +144,15 @@ typedef struct EvoAttnParams {
 
     /* Output gate of the Evoformer block, fused (all three NULL: no gate).  `gate` holds the gate
      * logits g, element for element like q (same dtype, same four strides).  evoattn_fwd then
-     * writes sigmoid(g) * O to o_gated (laid out like o) from its epilogue, in addition to the
-     * ungated O in `o`, which stays the tensor the backward takes delta = <dO, O> from.
-     * evoattn_bwd takes in `dout` the gradient of o_gated, forms dO = dout * sigmoid(g) and
-     * dgate = dout * O * sigmoid(g) * (1 - sigmoid(g)) in one pass over the rows (dgate laid out
-     * like q; dO goes to the workspace, laid out like q, which grows by q's extent in memory) and
-     * runs the attention backward on that dO.  The q-family may be dense or a slot of a buffer of
-     * up to 8 such tensors (Q, K, V and the gate as slices of one projection's result: strides of
-     * [B][S][N][W][H][D]), not sparser.  The reference returns O
+     * writes Og = sigmoid(g) * O to o_gated (laid out like o) from its epilogue; the ungated O goes
+     * to `o` as well if `o` is not NULL, and is not written at all if it is.  evoattn_bwd takes in
+     * `dout` the gradient of Og and in `o_gated` the forward's Og (or, with o_gated NULL, the
+     * ungated O in `o`), forms dO = dout * sigmoid(g), dgate = dout * Og * (1 - sigmoid(g)) and
+     * delta = rowsum(dout * Og) (= rowsum(dO * O)) in one pass over the rows (dgate laid out like
+     * q; dO goes to the workspace, laid out like q, which grows by q's extent in memory) and runs
+     * the attention backward on that dO and that delta: no ungated O is read.  The q-family may be
+     * dense or a slot of a buffer of up to 8 such tensors (Q, K, V and the gate as slices of one
+     * projection's result: strides of [B][S][N][W][H][D]), not sparser.  The reference returns O
      * ungated (evoformer.py:735); its callers apply the gate as a separate step. */
     const void *gate;
     void       *o_gated;

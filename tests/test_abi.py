@@ -28,7 +28,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert set(names) == set(_lib.EXPORTS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.evoattn_version() == 3
+    assert lib.evoattn_version() == 4
 
 
 def test_struct_layout_matches_header():
@@ -215,6 +215,16 @@ def test_gate_validation_on_the_host(lib):
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL        # no dgate
     p.dgate = fake
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == 0
+    # the gated output may stand alone (no ungated O is written, none is read); without a gate `o` is required
+    keep, p.o = p.o, None
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == 0
+    p.o_gated = None
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == _lib.EVO_EINVAL
+    p.o, p.o_gated = keep, fake
+    q = good()
+    q.o = None
+    assert lib.evoattn_check(ctypes.byref(q), _lib.EVO_PASS_FWD) == _lib.EVO_EINVAL
     q = good()
     need_plain = lib.evoattn_bwd_workspace_bytes(ctypes.byref(q))
     assert lib.evoattn_bwd_workspace_bytes(ctypes.byref(p)) >= need_plain + 1 * 4 * 64 * 2 * 32 * 2   # + dO, bf16

@@ -156,6 +156,6 @@ def test_gated_attention_compiles_without_a_graph_break(E):
     tests = ("test_schema", "test_faketensor", "test_autograd_registration")
     torch.library.opcheck(torch.ops.evoattn.fwd_gated, (q, k, v, m, b, g, False), test_utils=tests)
     with torch.no_grad():
-        og, o, lse, prep, seen = torch.ops.evoattn.fwd_gated(q, k, v, m, b, g, False)
+        og, lse, prep, seen = torch.ops.evoattn.fwd_gated(q, k, v, m, b, g, False)
     torch.library.opcheck(torch.ops.evoattn.bwd_gated, (x["dO"].to(dev), q.detach(), k.detach(), v.detach(), m, b.detach(), g.detach(),
-                                                        o, lse, prep, seen, False, True, False), test_utils=tests[:2])
+                                                        og, lse, prep, seen, False, True, False), test_utils=tests[:2])
