@@ -65,7 +65,14 @@ static int check_common(const EvoAttnParams *p) {
     if (!aligned(p->q, es) || !aligned(p->k, es) || !aligned(p->v, es) || !aligned(p->o, es) || !aligned(p->lse, 4))
         return EVO_EALIGN;
     if (p->bias && !aligned(p->bias, elem_size(p->bias_dtype))) return EVO_EALIGN;
-    if (p->gate && (!aligned(p->gate, 16) || !aligned(p->o_gated, 16))) return EVO_EALIGN;   // rows are moved in 8- and 16-byte pieces (o_gated may be NULL in a backward call)
+    if (p->gate) {
+        // The gate's kernels move rows in 8- and 16-byte pieces whichever attention kernels run: every tensor laid out
+        // like q starts on a 16-byte boundary and every stride is a whole number of such pieces (o_gated may be NULL
+        // in a backward call, o in any call).
+        const int64_t per16 = 16 / es;
+        if (p->stride_b % per16 || p->stride_h % per16 || p->stride_s % per16 || p->stride_n % per16) return EVO_EALIGN;
+        if (!aligned(p->gate, 16) || !aligned(p->o_gated, 16) || !aligned(p->o, 16)) return EVO_EALIGN;
+    }
     if (p->mask_kind == EVO_MASK_F32 && !aligned(p->mask, 4)) return EVO_EALIGN;
     if ((p->mask_kind == EVO_MASK_BF16 || p->mask_kind == EVO_MASK_F16) && !aligned(p->mask, 2)) return EVO_EALIGN;
     return EVO_OK;

@@ -80,8 +80,10 @@ enum {
 };
 #define EVO_FLAG_ALL (1 | 2 | 4 | 8 | 16 | 0x80 | 0x100 | 0x200 | 0x400 | 0x800 | 0x1000 | 0x2000)
 
-/* A problem (b, s) whose every key carries a mask value below this is a "dead row"; see lse below. */
-#define EVOATTN_SHIFT_THRESHOLD (-1.0e5f)
+/* A problem (b, s) whose every key carries a mask value below this is a "dead row"; see lse below.
+ * (An fp32 sum of such a mask value and a score of order one is the mask value: half a unit in the
+ * last place of 5e8 is 16.) */
+#define EVOATTN_SHIFT_THRESHOLD (-5.0e8f)
 
 /* error codes */
 enum {
@@ -103,10 +105,15 @@ enum { EVO_PASS_FWD = 0, EVO_PASS_BWD = 1 };
  * (evoformer.py:648-650) is (S*N*H*D, S*N*D, N*D, D); a true per-head view of the same
  * tensor is (S*N*H*D, D, N*H*D, H*D).
  * lse is dense [B][H][S][N] fp32.  For a problem whose every key carries a mask value
- * below EVOATTN_SHIFT_THRESHOLD (-1e5) the scores are the mask values alone, less the
- * largest of them (q.k and the bias are swamped by such a mask in fp32 arithmetic; the
- * shift cancels in O and in every gradient), and lse holds the log-sum-exp of those
- * shifted scores; otherwise lse = log sum_j exp(score_ij).
+ * below EVOATTN_SHIFT_THRESHOLD (-5e8: the reference's fill for a bool mask, an additive
+ * mask of -1e9) the scores are the mask values alone, less the largest of them (in the
+ * reference's fp32 arithmetic q.k and the bias vanish next to such a mask: equal mask
+ * values give uniform probabilities; the shift cancels in O and in every gradient), and
+ * lse holds the log-sum-exp of those shifted scores.  A row masked throughout by less
+ * (say -2e5) keeps q.k and the bias, rounded to the mask's last place as fp32 eager
+ * rounds them (there the two agree as far as that rounding lets them: 1.6e-2 in a score
+ * at -2e5).  Otherwise
+ * lse = log sum_j exp(score_ij).
  */
 typedef struct EvoAttnParams {
     int32_t B, S, N, H, D;
@@ -152,7 +159,9 @@ typedef struct EvoAttnParams {
      * q; dO goes to the workspace, laid out like q, which grows by q's extent in memory) and runs
      * the attention backward on that dO and that delta: no ungated O is read.  The q-family may be
      * dense or a slot of a buffer of up to 8 such tensors (Q, K, V and the gate as slices of one
-     * projection's result: strides of [B][S][N][W][H][D]), not sparser.  The reference returns O
+     * projection's result: strides of [B][S][N][W][H][D]), not sparser; with a gate every tensor
+     * laid out like q starts on a 16-byte boundary and the four strides are multiples of 16 bytes
+     * (else EVO_EALIGN: the gate's kernels move rows in 16-byte pieces).  The reference returns O
      * ungated (evoformer.py:735); its callers apply the gate as a separate step. */
     const void *gate;
     void       *o_gated;

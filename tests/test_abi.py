@@ -184,7 +184,7 @@ def test_every_flag_bit_is_declared_in_the_header(lib):
 def test_shift_threshold_is_the_header_constant():
     text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
     m = re.search(r"#define\s+EVOATTN_SHIFT_THRESHOLD\s+\((-[0-9.e]+)f\)", text)
-    assert m and float(m.group(1)) == -1.0e5
+    assert m and float(m.group(1)) == -5.0e8
     common = open(os.path.join(ROOT, "evoformer_triton_amd", "csrc", "common.h")).read()
     assert "kShiftThreshold = EVOATTN_SHIFT_THRESHOLD" in common
 
@@ -245,6 +245,13 @@ def test_gate_validation_on_the_host(lib):
     B, S, N, H, D = 1, 4, 64, 2, 32
     p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * H * D, D, N * H * D, H * D
     p.gate = p.o_gated = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    # strides that are no whole number of 16-byte pieces: the gate's kernels move rows in such pieces
+    p = good()
+    p.gate = p.o_gated = fake
+    p.stride_n += 2
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EALIGN
+    p.gate = p.o_gated = None                                    # without a gate such rows go to the kernels that read element by element
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
     # gate outputs without a gate are a mistake
     p = good()

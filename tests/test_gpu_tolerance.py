@@ -182,21 +182,20 @@ def test_dbias_of_small_gradients_on_the_per_problem_dq_kernel(E, scale_exp):
     assert torch.equal(small["dBias"], base["dBias"] * 2.0 ** scale_exp)
 
 
-def test_dead_row_rule_is_shared_by_both_kernel_families(E):
-    """A row whose every key carries an additive mask of -2e5 (below the shift threshold, yet
-    small enough that fp32 would keep some of q.k + bias next to it) with a large bias: the
-    matrix-core kernels and the fp32-arithmetic kernels, which may serve the forward and the
-    backward of one call, treat it alike (scores = the mask alone: uniform probabilities), so
-    either family's backward is normalised against either family's log-sum-exp."""
-    from evoformer_triton_amd import _lib
+def _masked_rows_case(fill):
     B, S, N, H, D = 1, 4, 96, 2, 32
     g = torch.Generator().manual_seed(5)
     x = {n: torch.randn((B, S, N, H, D), generator=g).to(torch.bfloat16) for n in ("Q", "K", "V", "dO")}
     mask = torch.zeros((B, S, 1, 1, N))
-    mask[0, 1] = -2.0e5
-    mask[0, 2, 0, 0, 40:] = -2.0e5
+    mask[0, 1] = fill
+    mask[0, 2, 0, 0, 40:] = fill
     x["mask"] = mask
     x["bias"] = (torch.randn((B, 1, H, N, N), generator=g) * 3.0)
+    return x
+
+
+def _both_families(E, x):
+    from evoformer_triton_amd import _lib
     out = {}
     for name, flags in (("mfma", 0), ("generic", _lib.EVO_FLAG_FORCE_GENERIC)):
         E.FLAGS = flags
@@ -204,6 +203,17 @@ def test_dead_row_rule_is_shared_by_both_kernel_families(E):
             out[name], _ = c_abi_fwd_bwd(E, x, dbias_fp32=True)
         finally:
             E.FLAGS = 0
+    return out
+
+
+def test_dead_row_rule_is_shared_by_both_kernel_families(E):
+    """A row whose every key carries an additive mask of -1e9 (below the shift threshold: in fp32 the
+    sum of such a mask and q.k + bias is the mask) with a large bias: the matrix-core kernels and the
+    fp32-arithmetic kernels, which may serve the forward and the backward of one call, treat it alike
+    (scores = the mask alone: uniform probabilities, as fp32 eager gives), so either family's backward
+    is normalised against either family's log-sum-exp."""
+    x = _masked_rows_case(-1.0e9)
+    out = _both_families(E, x)
     for n in ("O", "dQ", "dK", "dV", "dBias"):
         assert torch.isfinite(out["mfma"][n].float()).all() and torch.isfinite(out["generic"][n].float()).all()
         a, b = out["mfma"][n].float(), out["generic"][n].float()
@@ -214,3 +224,30 @@ def test_dead_row_rule_is_shared_by_both_kernel_families(E):
     # no gradient reaches Q or K of the dead row through uniform probabilities' scores ... but it does reach V
     dVh = eager.to_heads(out["generic"]["dV"].float().cpu())
     assert dVh[0, :, 1].abs().max() > 0
+    # and fp32 eager says the same of that row
+    want = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], compute_dtype=torch.float32)
+    for fam in ("mfma", "generic"):
+        for n in ("O", "dQ", "dK", "dV"):
+            got = eager.to_heads(out[fam][n].float().cpu())[0, :, 1]
+            ref = eager.to_heads(want[n].float())[0, :, 1]
+            assert bool(((got - ref).abs() <= TOL + 2.0 ** -8 * ref.abs()).all()), (fam, n, max_abs(got, ref))
+
+
+def test_a_row_masked_throughout_by_a_moderate_value_follows_fp32_eager(E):
+    """Every key of a row at -2e5: above the shift threshold, so q.k and the bias count, as they do in
+    fp32 eager, where they survive next to such a mask rounded to its last place (1.6e-2 at 2e5).  Both
+    kernel families against fp32 eager on that row; the allowance on top of the tolerance is what one
+    such rounding of a score does to a probability (e^0.0156 - 1) times the entry's scale."""
+    x = _masked_rows_case(-2.0e5)
+    out = _both_families(E, x)
+    want = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], compute_dtype=torch.float32)
+    Vh = eager.to_heads(x["V"].float())
+    for fam in ("mfma", "generic"):
+        for n in ("O", "dQ", "dK", "dV"):
+            got = eager.to_heads(out[fam][n].float().cpu())[0, :, 1]
+            ref = eager.to_heads(want[n].float())[0, :, 1]
+            assert torch.isfinite(got).all()
+            assert bool(((got - ref).abs() <= TOL + 1.6e-2 * max(1.0, float(ref.abs().max())) + 2.0 ** -8 * ref.abs()).all()), (fam, n, max_abs(got, ref))
+        # the row is not the mean of V: its probabilities follow q.k + bias
+        Oh = eager.to_heads(out[fam]["O"].float().cpu())
+        assert (Oh[0, :, 1] - Vh[0, :, 1].mean(1, keepdim=True)).abs().max() > 0.1
