@@ -574,7 +574,11 @@ class _SlotAttention(torch.autograd.Function):
 
     forward(P, res_mask, pair_bias, gated) -> (out, grad_slot): `out` is slot 1 (gated) or slot 0 as a
     [B,S,N,H,D] view, `grad_slot` is slot 2 as such a view, for the consumer to write the gradient of `out`
-    into (a gradient that arrives elsewhere is copied there).  backward returns DP, the gradient of P, whole:
+    into (a gradient that arrives elsewhere is copied there).  The backward uses slot 2 as its own memory: with
+    a gate it overwrites it with the gradient of the ungated output, so a consumer that hands `grad_slot` back
+    as the gradient of `out` must not read it again afterwards (a hook on `out`'s gradient that runs later, or
+    a second consumer of that gradient, would see dO * sigmoid(g)).  `out` is saved for the backward like any
+    output: changing it in place raises autograd's usual error.  backward returns DP, the gradient of P, whole:
     the projection's input and weight gradients are single GEMMs over it."""
 
     @staticmethod
@@ -595,36 +599,38 @@ class _SlotAttention(torch.autograd.Function):
                 p.o = None
                 p.gate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(OB[:, :, :, 1])
             _lib.check(lib.evoattn_fwd(ctypes.byref(p), _stream(P.device)), "evoattn_fwd")
-        ctx.save_for_backward(P, mask, bias, lse, prep)
-        # Not among the saved tensors, and under a version counter of its own (`.data`): the consumer writes the
-        # incoming gradient into slot 2 in place, which must not look like a change of `out` (the same memory
-        # object) to whoever saved `out` for its backward.
-        raw = OB.data
-        ctx.OB = raw
+        out = OB[:, :, :, 1 if gated else 0]
+        # `out` is what the backward reads (O, or with a gate sigmoid(g) * O): saved like any output, so that a
+        # consumer who changes it in place is told so by autograd's version check.  Slot 2 alone is kept under a
+        # version counter of its own (`.data`): the consumer writes the incoming gradient there in place, which
+        # must not look like a change of `out` (the same memory object) to whoever saved `out` for its backward.
+        grad_slot = OB.data[:, :, :, 2]
+        ctx.save_for_backward(P, mask, bias, lse, prep, out)
+        ctx.grad_slot = grad_slot
         ctx.gated = bool(gated)
         ctx.mask_meta = (mask_kind, mstr, None if res_mask is None else (tuple(res_mask.shape), res_mask.dtype))
         ctx.bias_meta = (bias_dt, bstr, None if pair_bias is None else (tuple(pair_bias.shape), pair_bias.dtype))
-        out, grad_slot = OB[:, :, :, 1 if gated else 0], raw[:, :, :, 2]
         ctx.mark_non_differentiable(grad_slot)
         ctx.set_materialize_grads(False)      # (no tensor of zeros for the second output's gradient, which nobody has)
         return out, grad_slot
 
     @staticmethod
     def _params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse):
+        """OB: the buffer of outputs (its slot 0 is O), or None where the caller sets `o` / `o_gated` itself."""
         B, S, N, W, H, D = P.shape
-        p = _params(P[:, :, :, 0], P[:, :, :, 1], P[:, :, :, 2], mask, mask_kind, mstr, bias, bias_dt, bstr, OB[:, :, :, 0], lse, "ds4sci")
+        p = _params(P[:, :, :, 0], P[:, :, :, 1], P[:, :, :, 2], mask, mask_kind, mstr, bias, bias_dt, bstr,
+                    None if OB is None else OB[:, :, :, 0], lse, "ds4sci")
         p.stride_b, p.stride_h, p.stride_s, p.stride_n = S * N * W * H * D, D, N * W * H * D, W * H * D
         return p
 
     @staticmethod
     def backward(ctx, dout, _unused):
         lib = _lib.load()
-        P, mask, bias, lse, prep = ctx.saved_tensors
-        OB = ctx.OB
+        P, mask, bias, lse, prep, out = ctx.saved_tensors
         B, S, N, W, H, D = P.shape
         mask_kind, mstr, mask_orig = ctx.mask_meta
         bias_dt, bstr, bias_orig = ctx.bias_meta
-        slot = OB[:, :, :, 2]
+        slot = ctx.grad_slot
         if dout is None:                      # the output took no part in what is differentiated
             return torch.zeros_like(P), None, None, None
         in_place = dout.data_ptr() == slot.data_ptr() and dout.dtype == slot.dtype and dout.shape == slot.shape and all(
@@ -635,12 +641,14 @@ class _SlotAttention(torch.autograd.Function):
         want_dbias = bool(ctx.needs_input_grad[2] and bias is not None)
         with _on_device(P.device):
             DP = torch.empty_like(P) if W == (4 if ctx.gated else 3) else torch.zeros_like(P)
-            p = _SlotAttention._params(P, OB, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
+            p = _SlotAttention._params(P, None, mask, mask_kind, mstr, bias, bias_dt, bstr, lse)
             p.dout, p.dq, p.dk, p.dv = _ptr(slot), _ptr(DP[:, :, :, 0]), _ptr(DP[:, :, :, 1]), _ptr(DP[:, :, :, 2])
             if ctx.gated:     # slot 2 is this Function's own memory: the gradient of the ungated output takes its place
-                p.o = None    # (delta and the gate's gradient come from the gated output, slot 1)
-                p.gate, p.dgate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(DP[:, :, :, 3]), _ptr(OB[:, :, :, 1])
+                # (delta and the gate's gradient come from the gated output, which is `out`; no ungated O exists)
+                p.gate, p.dgate, p.o_gated = _ptr(P[:, :, :, 3]), _ptr(DP[:, :, :, 3]), _ptr(out)
                 p.flags |= _lib.EVO_FLAG_GATE_DOUT_INPLACE
+            else:
+                p.o = _ptr(out)
             dbias = dmask = None
             if want_dbias:
                 dbias = torch.empty((B, H, N, N), device=P.device, dtype=bias.dtype)

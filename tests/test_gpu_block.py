@@ -276,6 +276,27 @@ def test_slot_attention_matches_the_dense_per_head_call(case, dtype):
     assert torch.equal(dP2, dP) and torch.equal(db2, db)
 
 
+@pytest.mark.parametrize("gated", [False, True], ids=["plain", "gated"])
+def test_slot_attention_output_changed_in_place_is_an_error(gated):
+    """The backward reads `out` (O, or with a gate sigmoid(g) * O): it is saved like any output, so a consumer
+    that changes it in place before the backward gets autograd's version error, not wrong gradients; writing
+    the gradient into `grad_slot`, the same memory object, is not such a change."""
+    import evoformer_triton_amd.evoformer as E
+    B, S, N, H, D = 1, 3, 64, 2, 32
+    W = 4 if gated else 3
+    dev = torch.device("cuda", torch.cuda.current_device())
+    g = torch.Generator().manual_seed(2)
+    P = torch.randn((B, S, N, W, H, D), generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    out, slot = E._SlotAttention.apply(P, None, None, gated)
+    slot.copy_(torch.randn((B, S, N, H, D), generator=g).to(torch.bfloat16).to(dev))
+    torch.autograd.grad(out, [P], slot, retain_graph=True)
+    with pytest.raises(RuntimeError, match="is a view and is being modified inplace"):
+        out.mul_(2.0)                      # (autograd refuses this for a view made inside a Function)
+    out.detach().mul_(2.0)                 # the same memory changed behind autograd's back: caught by the version check
+    with pytest.raises(RuntimeError, match="modified inplace|modified by an inplace operation"):
+        torch.autograd.grad(out, [P], slot)
+
+
 def test_block_takes_the_slot_path_on_the_gpu():
     """In 16-bit on the GPU the block's Q, K, V and gate come from one GEMM and reach the kernels as slots;
     the layer-by-layer path (fp32, under the tracer) gives the same to the rounding of the dtype."""
