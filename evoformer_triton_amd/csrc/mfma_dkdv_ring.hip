@@ -379,7 +379,12 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
         if (active) {
             if (want_dm) {
                 dm += __shfl_xor(dm, 32);
-                if (g == 0 && key < p.N) e.dmask_part[row0 + key] = dm;
+                // (a buffer store: the row's address is scalar and the lane adds its key, formed here from the lane
+                // number: an address or an offset per lane kept across the rows would be one or two registers spilled)
+                const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)(e.dmask_part + row0), 0, p.N * 4, 0x00020000);
+                unsigned ln;
+                asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+                if (g == 0 && key < p.N) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dm), rs, (int)((key0 + (ln & 31)) * 4), 0, 0);
             }
             if (key < p.N) {
                 T *dK = (T *)p.dk + base + (int64_t)key * sn;
