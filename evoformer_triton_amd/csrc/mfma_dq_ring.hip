@@ -461,6 +461,14 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
+                    // The two waves of a SIMD (w and w + 4) take turns at the higher issue priority, tile by tile
+                    // (S = 512, N = 256, H = 8, head dim 32: 2 us of 145 less).  Only where a wave has two tiles per
+                    // stage: with one, the turn would leave the younger wave ahead throughout, and the older one, which
+                    // also sums the partial dQ, then ends its row late (rows of 384 and 768 keys: 8 % slower).
+                    if (NBLK == 1 && TPW == 2) {
+                        if (((jj ^ (wave >> 2)) & 1) != 0) __builtin_amdgcn_s_setprio(1);
+                        else __builtin_amdgcn_s_setprio(0);
+                    }
                     const int tb = jj * KQ + kq;         // tile inside the stage
                     const int kt = blk * TPB + tb;
                     if (MID && jj == TPW - 1) {
