@@ -280,14 +280,15 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     bool stage_dead = PRESCALE && uniform_load(e.dead + b * p.S + s_begin) != 0;
     auto stash_part = [&](const Staged &stg, int t, int i0, int i1, int par) {   // par: the buffer of stage t, t & 1
         const int blk = t % NBLK;
-        const int ninst = t >= T_total ? 0 : blk == 0 ? R::I_ALL : R::I_KVA;
+        if (t >= T_total) return;   // uniform (one branch for the stage, none per piece where every wave has all its pieces)
+        const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
         unsigned char *buf = lds + par * R::BUF_BYTES;
         const float cq = stage_dead ? 0.0f : cs;   // (the flag of the row this stage belongs to)
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             if (i < i0 || i >= i1) continue;
             const int n = wave + 8 * i;
-            if (n < ninst) {
+            if ((NBLK == 1 && 8 * i + 7 < R::I_ALL) || n < ninst) {
                 const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
                 if (n >= 2 * R::I_K && n < R::I_KVA)   // of a mask chunk (hi, mid, lo, 1, 1, 1, 0, 0) the first 8 bytes
                     *reinterpret_cast<uint2 *>(buf + dst + lane * 8) = make_uint2(stg.v[i][0], stg.v[i][1]);
@@ -297,7 +298,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg.v[i];
             }
         }
-        if (i1 >= IPW && wave == 0 && blk == 0 && t < T_total && lane < QR) {
+        if (i1 >= IPW && wave == 0 && blk == 0 && lane < QR) {
             *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-stg.lse * kLog2e);
             if (e.delta_given) *reinterpret_cast<float *>(buf + R::OFF_DL + lane * 4) = stg.dl;
         }
