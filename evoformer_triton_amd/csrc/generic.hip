@@ -333,7 +333,7 @@ int launch_delta_generic(const EvoAttnParams &p, const Extra &e, hipStream_t st)
 // given, ungated (p.o),
 //     dO    = dout * sigmoid(g)                           -> dout_ungated (what the attention backward runs on)
 //     dg    = dout * Og * (1 - sigmoid(g))                -> p.dgate       (= dout * O * sigmoid(g) * (1 - sigmoid(g)))
-//     delta = sum over the head dim of dout * Og          -> delta         (= rowsum(dO * O), from unrounded products)
+//     delta = sum over the head dim of dO * (Og / sigmoid(g)) -> delta      (= rowsum(dO * O), with dO as stored)
 // the first two laid out like q, delta [B][H][S][N].  With delta formed here the dQ kernels need no
 // ungated O, so the forward need not write one.  One thread per 8 consecutive head-dim elements of
 // one row at a time; the D / 8 threads of a row are neighbours in a wave and add their parts of delta.
@@ -379,12 +379,16 @@ __global__ void __launch_bounds__(256) gate_bwd_kernel(EvoAttnParams p, T *dout_
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 // (the 16-bit types take the hardware's exp2 and reciprocal, one ulp each, as the MFMA forward does)
-                const float sg = sizeof(T) == 4 ? 1.0f / (1.0f + expf(-(float)b2[j])) : sigmoidf((float)b2[j]);
+                const float den = 1.0f + (sizeof(T) == 4 ? expf(-(float)b2[j]) : fast_exp2(-(float)b2[j] * kLog2e));
+                const float sg = sizeof(T) == 4 ? 1.0f / den : __builtin_amdgcn_rcpf(den);
                 const float gr = (float)a[j];
                 const float og = FROM_GATED ? (float)c2[j] : (float)c2[j] * sg;   // sigmoid(g) * O
                 r_o[j] = (T)(gr * sg);
                 r_g[j] = (T)(gr * og * (1.0f - sg));
-                dsum = fmaf(gr, og, dsum);
+                // delta from the dO that the attention backward will read, rounded as it is stored, against
+                // O = Og / sigmoid(g): dP is formed from the same rounded dO, and in dS = P (dP - delta) the
+                // rounding of dO then cancels as far as P is peaked (with delta from dout * Og it does not)
+                dsum = fmaf((float)r_o[j], FROM_GATED ? (float)c2[j] * den : (float)c2[j], dsum);
             }
             if (i0 < total) {
                 *reinterpret_cast<vec *>(d_o + j0) = r_o;

@@ -155,7 +155,7 @@ typedef struct EvoAttnParams {
      * to `o` as well if `o` is not NULL, and is not written at all if it is.  evoattn_bwd takes in
      * `dout` the gradient of Og and in `o_gated` the forward's Og (or, with o_gated NULL, the
      * ungated O in `o`), forms dO = dout * sigmoid(g), dgate = dout * Og * (1 - sigmoid(g)) and
-     * delta = rowsum(dout * Og) (= rowsum(dO * O)) in one pass over the rows (dgate laid out like
+     * delta = rowsum(dO * Og / sigmoid(g)) (= rowsum(dO * O)) in one pass over the rows (dgate laid out like
      * q; dO goes to the workspace, laid out like q, which grows by q's extent in memory) and runs
      * the attention backward on that dO and that delta: no ungated O is read.  The q-family may be
      * dense or a slot of a buffer of up to 8 such tensors (Q, K, V and the gate as slices of one
