@@ -390,6 +390,11 @@ static bool kv_ring_ok(const EvoAttnParams &p) {
     return !p.bias || p.bias_dtype == p.dtype;
 }
 
+// whether dQ of this call comes from the kernel over a chunk of rows in the form that also does the gate's pass
+static bool gate_in_dq(const EvoAttnParams &p) {
+    return mfma_ok(p, EVO_PASS_BWD) && !dq_split_ok(p) && !dq_wide_ok(p) && dq_ring_ok(p) && mfma_dqr_gate_ok(p.D, p.N);
+}
+
 static int launch_dq(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     if (dq_split_ok(p)) {
         EvoAttnParams q = p;
@@ -472,21 +477,32 @@ int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
     // gradient of the ungated output (into the workspace) and of the gate, and the attention
     // backward below runs on the former.
     EvoAttnParams ungated = *p0;
+    Extra e{};
     if (p0->gate) {
         // (in place: a thread reads its 8 elements of dout before it writes them)
         void *d_o = (p0->flags & EVO_FLAG_GATE_DOUT_INPLACE) ? const_cast<void *>(p0->dout) : (void *)(ws + w.dout_ungated);
-        if ((rc = launch_gate_bwd(*p0, d_o, (float *)(ws + w.delta), st))) return rc;
         ungated.dout = d_o;
         ungated.gate = nullptr;
         ungated.o_gated = nullptr;
+        ungated.dgate = nullptr;
+        // Where dQ comes from the kernel over a chunk of rows in its form for up to 256 keys at head dim 32, that
+        // kernel does the gate's pass on the rows it stages anyway (it runs before the dK/dV kernel, which reads
+        // the gradient of the ungated output it writes).
+        if (gate_in_dq(ungated) && p0->o_gated && !(p0->flags & EVO_FLAG_ONLY_DKDV)) {
+            e.gate_dout = p0->dout;
+            e.gate_logits = p0->gate;
+            e.gate_og = p0->o_gated;
+            e.gate_dgate = p0->dgate;
+        } else if ((rc = launch_gate_bwd(*p0, d_o, (float *)(ws + w.delta), st))) {
+            return rc;
+        }
     }
     const EvoAttnParams *p = &ungated;
-    Extra e{};
     e.n_chunks = w.n_chunks;
     e.chunk = w.chunk;
     e.vec_ok = bias_vec_ok(*p);
     e.delta = (float *)(ws + w.delta);
-    e.delta_given = p0->gate ? 1 : 0;   // (the gate's pass wrote it; the dQ kernels then read no ungated O)
+    e.delta_given = p0->gate && !e.gate_dout ? 1 : 0;   // (the gate's pass wrote it; the dQ kernels then read no ungated O)
     e.shift = (float *)(ws + w.shift);
     e.dmask_part = (float *)(ws + w.dmask_part);
     e.dbias_part = (float *)(ws + w.dbias_part);

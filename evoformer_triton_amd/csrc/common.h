@@ -39,6 +39,13 @@ struct Extra {
     int bias_direct;   // the one-workgroup-per-problem kernels read the bias from the caller's tensor, not from bq / bk
     int dbias_chunks;  // > 0: the dK/dV kernel over a chunk of rows also sums that many dBias partials (else `dbias_reduce` does)
     int delta_given;   // `delta` already holds rowsum(dO * O) (the gate's pass wrote it): the dQ kernels read it and do not touch o
+    // The gate's backward inside the dQ kernel over a chunk of rows (gate_dout non-null): that kernel stages the
+    // gradient of the gated output, the gate's logits and the gated output, writes the gradient of the ungated
+    // output to p.dout (for the dK/dV kernel) and the gate's gradient, and forms delta, as the gate's pass would.
+    const void *gate_dout;   // gradient of the gated output, laid out like q
+    const void *gate_logits;
+    const void *gate_og;     // sigmoid(g) * O as the forward saved it
+    void *gate_dgate;
     float *delta;      // [B][H][S][N]
     float *shift;      // [B][S] per-row mask shift (plain kernels)
     float *dbias_part; // [n_chunks][B][H][N][N]

@@ -99,7 +99,14 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 #define EVO_TR(slot) do {} while (0)
 #endif
 
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB>
+// GATE: the gate's backward pass on the rows the kernel stages (the form of one stage of up to 256 keys at head
+// dim 32): in place of dO and O the workgroup asks for the gradient of the gated output, the gate's logits and
+// the gated output of its 64 query rows; the wave that holds a 1 KB piece of all three forms, as the gate's pass
+// of its own does (generic.hip) and bit for bit like it, dO = dout * sigmoid(g) (to the stage, and to p.dout for
+// the dK/dV kernel), dgate = dout * Og * (1 - sigmoid(g)) and delta = rowsum(dO * Og / sigmoid(g)) (to the
+// stage and to e.delta).  Pieces 36..39 are then dout, 40..43 Q, 44..47 the logits, 52..55 Og (a piece and
+// the two that follow it 8 and 16 numbers later belong to the same wave), 48..51 are not used.
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false>
 __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef RingGeo<D, QT, KB> R;
@@ -172,7 +179,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // list of 1 KB pieces (64 lanes x 16 bytes); piece n belongs to wave n % 8.  Lane i of
     // piece m of a row-major block fills LDS slot 64 m + i of that block, which the swizzle
     // assigns to some chunk of some row.
-    constexpr int IPW = (R::I_ALL + 7) / 8;   // most pieces one wave moves per stage
+    static_assert(!GATE || (NBLK == 1 && QT == 2 && KB == 256 && D == 32), "the gate's pass is built into one form");
+    constexpr int I_ALL = GATE ? R::I_KVA + 5 * R::I_Q : R::I_ALL;   // pieces of a stage with query rows
+    constexpr int IPW = (I_ALL + 7) / 8;   // most pieces one wave moves per stage
     struct Staged {
         u32x4 v[IPW];
         float lse;
@@ -189,7 +198,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         unsigned lane_off;
         int dst;
     };
-    auto describe = [&](int n, int blk) {
+    auto describe = [&](int n, int blk) __attribute__((always_inline)) {
         Piece d;
         if (n >= 2 * R::I_K && n < R::I_KVA) {
             const int m = n - 2 * R::I_K;
@@ -202,6 +211,14 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             int m, row0, off;
             if (n < R::I_K) { base = (const T *)p.k; m = n; row0 = blk * BKV; off = 0; }
             else if (n < 2 * R::I_K) { base = (const T *)p.v; m = n - R::I_K; row0 = blk * BKV; off = R::OFF_V; }
+            else if (GATE) {
+                const int kind = (n - R::I_KVA) / R::I_Q;   // dout, Q, logits, (unused: Q once more), Og
+                m = (n - R::I_KVA) % R::I_Q; row0 = qbase; off = R::OFF_Q;
+                if (kind == 0) { base = (const T *)e.gate_dout; off = R::OFF_G; }
+                else if (kind == 2) base = (const T *)e.gate_logits;
+                else if (kind == 4) base = (const T *)e.gate_og;
+                else base = (const T *)p.q;
+            }
             else if (n < R::I_KVA + R::I_Q) { base = (const T *)p.q; m = n - R::I_KVA; row0 = qbase; off = R::OFF_Q; }
             else if (n < R::I_KVA + 2 * R::I_Q) { base = (const T *)p.dout; m = n - R::I_KVA - R::I_Q; row0 = qbase; off = R::OFF_G; }
             else {   // (where delta is given there may be no ungated O: the piece is dO once more, and is not used)
@@ -223,7 +240,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     Piece fixed[NBLK == 1 ? IPW : 1];
     if (NBLK == 1) {
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) fixed[i] = describe(min(wave + 8 * i, R::I_ALL - 1), 0);
+        for (int i = 0; i < IPW; ++i) fixed[i] = describe(min(wave + 8 * i, I_ALL - 1), 0);
     }
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
@@ -245,10 +262,10 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         flse += p.N;
     };
     // pieces [i0, i1) of stage t; the last piece takes the log-sum-exp along
-    auto fetch_part = [&](Staged &stg, int t, int i0, int i1) {
+    auto fetch_part = [&](Staged &stg, int t, int i0, int i1) __attribute__((always_inline)) {
         t = min(t, T_total - 1);
         const int row = t / NBLK, blk = t % NBLK;
-        const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
+        const int ninst = blk == 0 ? I_ALL : R::I_KVA;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             if (i < i0 || i >= i1) continue;
@@ -267,7 +284,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             const float *lsrc = NBLK == 1 ? flse : p.lse + lrow;
             stg.lse = lsrc[flse_off];
             // (delta has the layout of the log-sum-exp: the same offset from its own base)
-            if (e.delta_given) stg.dl = (e.delta + (lsrc - p.lse))[flse_off];
+            if (!GATE && e.delta_given) stg.dl = (e.delta + (lsrc - p.lse))[flse_off];
         }
     };
     auto fetch = [&](Staged &stg, int t) { fetch_part(stg, t, 0, IPW); };
@@ -278,29 +295,66 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     // for a row with every key masked, and the log-sum-exp as its three operand columns.
     constexpr bool PRESCALE = !G::RESID;
     bool stage_dead = PRESCALE && uniform_load(e.dead + b * p.S + s_begin) != 0;
-    auto stash_part = [&](const Staged &stg, int t, int i0, int i1, int par) {   // par: the buffer of stage t, t & 1
+    auto stash_part = [&](const Staged &stg, int t, int i0, int i1, int par) __attribute__((always_inline)) {   // par: the buffer of stage t, t & 1
         const int blk = t % NBLK;
         if (t >= T_total) return;   // uniform (one branch for the stage, none per piece where every wave has all its pieces)
-        const int ninst = blk == 0 ? R::I_ALL : R::I_KVA;
+        const int ninst = blk == 0 ? I_ALL : R::I_KVA;
         unsigned char *buf = lds + par * R::BUF_BYTES;
         const float cq = stage_dead ? 0.0f : cs;   // (the flag of the row this stage belongs to)
 #pragma unroll
         for (int i = 0; i < IPW; ++i) {
             if (i < i0 || i >= i1) continue;
             const int n = wave + 8 * i;
-            if ((NBLK == 1 && 8 * i + 7 < R::I_ALL) || n < ninst) {
+            if ((NBLK == 1 && 8 * i + 7 < I_ALL) || n < ninst) {
                 const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
-                if (n >= 2 * R::I_K && n < R::I_KVA)   // of a mask chunk (hi, mid, lo, 1, 1, 1, 0, 0) the first 8 bytes
+                const int qkind = GATE && n >= R::I_KVA ? (n - R::I_KVA) / R::I_Q : -1;   // (GATE: dout, Q, logits, unused, Og)
+                if (n >= 2 * R::I_K && n < R::I_KVA) {   // of a mask chunk (hi, mid, lo, 1, 1, 1, 0, 0) the first 8 bytes
                     *reinterpret_cast<uint2 *>(buf + dst + lane * 8) = make_uint2(stg.v[i][0], stg.v[i][1]);
-                else if (PRESCALE && n >= R::I_KVA && n < R::I_KVA + R::I_Q)
+                } else if (GATE && qkind == 0) {
+                    // the gate's pass on this lane's 8 elements of one query row (generic.hip: gate_bwd_kernel)
+                    if constexpr (GATE) {
+                        const v8 a = __builtin_bit_cast(v8, stg.v[i]), gl = __builtin_bit_cast(v8, stg.v[i + 1 < IPW ? i + 1 : i]),
+                                 og = __builtin_bit_cast(v8, stg.v[i + 2 < IPW ? i + 2 : i]);
+                        v8 r_o, r_g;
+                        float dsum = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float den = 1.0f + fast_exp2(-(float)gl[j] * kLog2e);
+                            const float sg = __builtin_amdgcn_rcpf(den);
+                            const float gr = (float)a[j], ogf = (float)og[j];
+                            r_o[j] = (T)(gr * sg);
+                            r_g[j] = (T)(gr * ogf * (1.0f - sg));
+                            dsum = fmaf((float)r_o[j], ogf * den, dsum);
+                        }
+                        // the C lanes of a row are neighbours (the swizzle permutes their chunks in pairs and pairs of pairs)
+#pragma unroll
+                        for (int w = 1; w < C; w <<= 1) dsum += __shfl_xor(dsum, w);
+                        *reinterpret_cast<v8 *>(buf + dst + lane * 16) = r_o;
+                        const int L = (n - R::I_KVA) % R::I_Q * 64 + lane;
+                        const int r = L / C;
+                        if (L % C == 0) *reinterpret_cast<float *>(buf + R::OFF_DL + r * 4) = dsum;
+                        if (qbase + r < p.N) {
+                            // (the piece's element offset inside the tensors laid out like q: the row's, plus the lane's)
+                            const int64_t goff = base0 + (int64_t)t * p.stride_s;
+                            unsigned char *o_row = reinterpret_cast<unsigned char *>((T *)p.dout + goff) + fixed[i].lane_off;
+                            unsigned char *g_row = reinterpret_cast<unsigned char *>((T *)e.gate_dgate + goff) + fixed[i].lane_off;
+                            *reinterpret_cast<v8 *>(o_row) = r_o;
+                            *reinterpret_cast<v8 *>(g_row) = r_g;
+                            if (L % C == 0) e.delta[((int64_t)bh * p.S + s_begin + t) * p.N + qbase + r] = dsum;
+                        }
+                    }
+                } else if (GATE && qkind >= 2) {
+                    // (logits, Og: used above; the unused piece)
+                } else if (PRESCALE && (GATE ? qkind == 1 : n >= R::I_KVA && n < R::I_KVA + R::I_Q)) {
                     *reinterpret_cast<v8 *>(buf + dst + lane * 16) = scaled8<T>(__builtin_bit_cast(v8, stg.v[i]), cq);
-                else
+                } else {
                     *reinterpret_cast<u32x4 *>(buf + dst + lane * 16) = stg.v[i];
+                }
             }
         }
         if (i1 >= IPW && wave == 0 && blk == 0 && lane < QR) {
             *reinterpret_cast<uint2 *>(buf + R::OFF_L + lane * 8) = pack_split3<T>(-stg.lse * kLog2e);
-            if (e.delta_given) *reinterpret_cast<float *>(buf + R::OFF_DL + lane * 4) = stg.dl;
+            if (!GATE && e.delta_given) *reinterpret_cast<float *>(buf + R::OFF_DL + lane * 4) = stg.dl;
         }
     };
     auto stash = [&](const Staged &stg, int t, int par) { stash_part(stg, t, 0, IPW, par); };
@@ -431,10 +485,12 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                         const int o = R::swz(qi * 32 + li, 2 * ks + g);
                         const v8 qraw = *reinterpret_cast<const v8 *>(buf + R::OFF_Q + o);
                         gf[ks] = *reinterpret_cast<const v8 *>(buf + R::OFF_G + o);
-                        const v8 oraw = *reinterpret_cast<const v8 *>(buf + R::OFF_O + o);
                         if (PRESCALE) qf[ks] = qraw;   // scaled (and zeroed for a dead row) when it was staged
                         else if (!dead) scaled_hilo8<T>(qraw, cs, qf[ks], qlo[ks < KSD ? ks : 0]);
-                        dpart = dot8<T>(gf[ks], oraw, dpart);
+                        if constexpr (!GATE) {   // (with the gate's pass delta lies in the stage, and there is no O)
+                            const v8 oraw = *reinterpret_cast<const v8 *>(buf + R::OFF_O + o);
+                            dpart = dot8<T>(gf[ks], oraw, dpart);
+                        }
                     }
                 }
                 float dl;
@@ -443,7 +499,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
                     auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
                     dl = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
                 }
-                if (e.delta_given) dl = *reinterpret_cast<const float *>(buf + R::OFF_DL + (qi * 32 + li) * 4);   // uniform
+                if (GATE || e.delta_given) dl = *reinterpret_cast<const float *>(buf + R::OFF_DL + (qi * 32 + li) * 4);   // uniform
                 else if (kq == 0 && g == 0 && q0 + li < p.N) e.delta[pr.row0 + q0 + li] = dl;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
@@ -616,11 +672,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false>
 static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     typedef RingGeo<D, QT, KB> R;
     static PerDevice done{};
-    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB>;
+    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB, GATE>;
     if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, nullptr)) return rc;
     const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
     const unsigned grid = (unsigned)NQP * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
@@ -661,6 +717,12 @@ static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     if constexpr (D == 64) {
         if (f.nblk == 1) return dqr_launch<T, D, HAS_BIAS, 1, 2, 128>(p, e, st);
     } else {
+        if constexpr (D == 32) {
+            static_assert(dqr_form<32>(256).nblk == 1 && dqr_form<32>(256).qt == 2 && dqr_form<32>(256).kb == 256, "the form with the gate's pass");
+            if (e.gate_dout) return mfma_dqr_gate_ok(D, p.N) ? dqr_launch<T, D, HAS_BIAS, 1, 2, 256, true>(p, e, st) : EVO_EINVAL;
+        } else if (e.gate_dout) {
+            return EVO_EINVAL;   // (the caller asks for the gate's pass only where this kernel has it)
+        }
         if (f.nblk == 1 && f.kb == 256) return dqr_launch<T, D, HAS_BIAS, 1, 2, 256>(p, e, st);
         if constexpr (D == 8) {
             if (f.nblk == 1 && f.kb == 384) return dqr_launch<T, D, HAS_BIAS, 1, 2, 384>(p, e, st);

@@ -17,7 +17,7 @@ def E(gpu_device):
     return E
 
 
-def run_gated(E, x, gate, layout="reference", flags=0):
+def run_gated(E, x, gate, layout="reference", flags=0, bwd_flags=None):
     dev = torch.device("cuda", torch.cuda.current_device())
     q, k, v = (x[n].to(dev).requires_grad_() for n in "QKV")
     b = x["bias"].to(dev).requires_grad_()
@@ -25,6 +25,8 @@ def run_gated(E, x, gate, layout="reference", flags=0):
     E.FLAGS = flags
     try:
         og = E.evoformer_attention(q, k, v, x["mask"].to(dev), b, layout=layout, gate=g)
+        if bwd_flags is not None:
+            E.FLAGS = bwd_flags
         og.backward(x["dO"].to(dev))
     finally:
         E.FLAGS = 0
@@ -74,6 +76,26 @@ def test_gated_attention_fp32_check_mode_and_forced_generic(E):
     refb = eager.attention_fwd_bwd(xb["Q"], xb["K"], xb["V"], xb["mask"], xb["bias"], xb["dO"], compute_dtype=torch.float32,
                                    gate=gate.to(torch.bfloat16))
     check(run_gated(E, xb, gate.to(torch.bfloat16), flags=_lib.EVO_FLAG_FORCE_GENERIC), refb, 2e-2, "bf16 plain kernels")
+
+
+@pytest.mark.parametrize("layout", ["reference", "ds4sci"])
+def test_gate_pass_inside_the_dq_kernel_is_the_pass_of_its_own(E, layout):
+    """Rows of up to 256 keys at head dim 32 with a dBias to sum: the dQ kernel over a chunk of rows does the gate's
+    backward pass on the rows it stages.  The same call on the one-workgroup-per-problem kernels runs the pass as a
+    kernel of its own: the gate's gradient is the same bits (the same arithmetic in the same order), the other
+    gradients agree as those two kernel families do."""
+    from evoformer_triton_amd import _lib
+    shape = (1, 9, 251, 2, 32)
+    x = eager.make_inputs("C2", shape=shape, seed=33)
+    gate = (torch.randn(shape, generator=torch.Generator().manual_seed(6)) * 2.0).to(torch.bfloat16)
+    fused = run_gated(E, x, gate, layout)
+    apart = run_gated(E, x, gate, layout, bwd_flags=_lib.EVO_FLAG_PER_PROBLEM)   # (the same forward: the same saved output)
+    assert torch.equal(fused["Og"], apart["Og"]) and torch.equal(fused["dGate"], apart["dGate"])
+    for n in ("dQ", "dK", "dV", "dBias"):
+        assert (fused[n].float() - apart[n].float()).abs().max().item() <= 2e-2, n
+    ref = eager.attention_fwd_bwd(x["Q"], x["K"], x["V"], x["mask"], x["bias"], x["dO"], layout=layout,
+                                  compute_dtype=torch.float32, gate=gate)
+    check(fused, ref, 2e-2, f"{shape} {layout}")
 
 
 def test_gated_rows_of_one_key(E):
