@@ -47,7 +47,7 @@ static int check_common(const EvoAttnParams *p) {
         // The gate is read and its products written element for element like q; the backward keeps the gradient
         // of the ungated output in the workspace, laid out like q, gaps included: the q-family may be dense or a
         // slot of a buffer of up to 8 such tensors (Q, K, V and the gate as one projection's result), not sparser.
-        if (p->D % 8) return EVO_EUNSUPPORTED;
+        if (p->D % 8 || p->H > 256) return EVO_EUNSUPPORTED;   // (the gate's backward pass keeps 128 bytes of LDS per head)
         if (q_span(*p) > 8 * (int64_t)p->B * p->H * p->S * p->N * p->D) return EVO_EUNSUPPORTED;
     } else if (p->o_gated || p->dgate) {
         return EVO_EINVAL;

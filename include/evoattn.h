@@ -161,7 +161,7 @@ typedef struct EvoAttnParams {
      * dense or a slot of a buffer of up to 8 such tensors (Q, K, V and the gate as slices of one
      * projection's result: strides of [B][S][N][W][H][D]), not sparser; with a gate every tensor
      * laid out like q starts on a 16-byte boundary and the four strides are multiples of 16 bytes
-     * (else EVO_EALIGN: the gate's kernels move rows in 16-byte pieces).  The reference returns O
+     * (else EVO_EALIGN: the gate's kernels move rows in 16-byte pieces), and H is at most 256.  The reference returns O
      * ungated (evoformer.py:735); its callers apply the gate as a separate step. */
     const void *gate;
     void       *o_gated;

@@ -253,6 +253,11 @@ def test_gate_validation_on_the_host(lib):
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EALIGN
     p.gate = p.o_gated = None                                    # without a gate such rows go to the kernels that read element by element
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    # more heads than the gate's backward pass has LDS for
+    p = good(H=257)
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    p.gate = p.o_gated = fake
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == _lib.EVO_EUNSUPPORTED
     # gate outputs without a gate are a mistake
     p = good()
     p.dgate = fake
