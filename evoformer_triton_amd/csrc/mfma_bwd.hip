@@ -448,6 +448,10 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
         for (int r = 0; r < 16; ++r) dk[dt][r] = dv[dt][r] = 0.0f;
     float dm = 0.0f;
 
+    const int row_valid = (int)(((int64_t)(p.N - 1) * sn + D) * 2);   // bytes from a problem's first row to the end of its last
+    const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc((void *)Q, 0, row_valid, 0x00020000);
+    const __amdgpu_buffer_rsrc_t grs = __builtin_amdgcn_make_buffer_rsrc((void *)Gd, 0, row_valid, 0x00020000);
+    const int sn2 = (int)sn * 2;
     auto stage = [&](int qs0) {
         EVO_TK(1);
         __syncthreads();
@@ -455,21 +459,22 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
         // all loads first, then the conversions and LDS writes: one round trip, not one per piece
         constexpr int NIT = (srows * C + NTH - 1) / NTH;
         v8 qv[NIT], gv[NIT];
+        // (buffer loads: 32-bit lane offsets from the problem's first row; a row at or beyond N lies past the end of
+        // the resource and reads as zero)
 #pragma unroll
         for (int i = 0; i < NIT; ++i) {
             const int it = tid + i * NTH;
-            const int row = min(it / C, srows - 1), ch = it % C, qq = min(qs0 + row, p.N - 1);
-            qv[i] = ld8(Q + (int64_t)qq * sn + ch * 8);
-            gv[i] = ld8(Gd + (int64_t)qq * sn + ch * 8);
+            const int row = min(it / C, srows - 1), ch = it % C, off = (qs0 + row) * sn2 + ch * 16;
+            qv[i] = __builtin_bit_cast(v8, __builtin_amdgcn_raw_buffer_load_b128(qrs, off, 0, 0));
+            gv[i] = __builtin_bit_cast(v8, __builtin_amdgcn_raw_buffer_load_b128(grs, off, 0, 0));
         }
 #pragma unroll
         for (int i = 0; i < NIT; ++i) {
             const int it = tid + i * NTH;
             if (it < srows * C) {
                 const int row = it / C, ch = it % C;
-                const bool in = qs0 + row < p.N;
-                const v8 a = in ? qv[i] : zero8<T>();
-                const v8 bb2 = in ? gv[i] : zero8<T>();
+                const v8 a = qv[i];
+                const v8 bb2 = gv[i];
                 // the score operand carries scale*log2(e), rounded exactly as in the forward
                 v8 hi, lo;
                 scaled_hilo8<T>(a, cs, hi, lo);

@@ -155,11 +155,18 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
         }
     };
 
+    // K and V rows are buffer loads: a resource (in scalar registers) that describes the problem's K or V rows and a
+    // 32-bit byte offset per lane.  Rows at or beyond N lie past the end of the resource and read as zero (such keys
+    // carry the mask floor), so no lane tests its row, and no 64-bit address per lane lives across the stages.
+    const int kv_valid = (int)(((int64_t)(p.N - 1) * sn + D) * 2);   // bytes from the first K (V) row to the end of the last
+    const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc((void *)K, 0, kv_valid, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc((void *)V, 0, kv_valid, 0x00020000);
+    const int sn2 = (int)sn * 2;
     auto stage = [&](int kv0) {
         __syncthreads();  // readers of the previous stage are done
         for (int it = tid; it < BKV * (D / 8); it += NTH) {
             const int key = it / (D / 8), ch = it % (D / 8), kk = kv0 + key;
-            v8 val = kk < p.N ? ld8(K + (int64_t)kk * sn + ch * 8) : zero8<T>();
+            const v8 val = __builtin_bit_cast(v8, __builtin_amdgcn_raw_buffer_load_b128(krs, kk * sn2 + ch * 16, 0, 0));
             *reinterpret_cast<v8 *>(&Ks[key * KP + ch * 8]) = val;
         }
         for (int key = tid; key < BKV; key += NTH)   // (mask hi, mid, lo, 1, 1, 1, 0, 0); the floor past the padded N
@@ -167,8 +174,8 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_f
         constexpr int NPAIR = BKV / 2;
         for (int it = tid; it < NPAIR * (D / 8); it += NTH) {
             const int ch = it / NPAIR, jp = it % NPAIR, k0 = kv0 + 2 * jp;
-            v8 a = k0 < p.N ? ld8(V + (int64_t)k0 * sn + ch * 8) : zero8<T>();
-            v8 b = k0 + 1 < p.N ? ld8(V + (int64_t)(k0 + 1) * sn + ch * 8) : zero8<T>();
+            const v8 a = __builtin_bit_cast(v8, __builtin_amdgcn_raw_buffer_load_b128(vrs, k0 * sn2 + ch * 16, 0, 0));
+            const v8 b = __builtin_bit_cast(v8, __builtin_amdgcn_raw_buffer_load_b128(vrs, (k0 + 1) * sn2 + ch * 16, 0, 0));
             const int pos = perm_pos(2 * jp);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
