@@ -235,28 +235,28 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
         }
         return d;
     };
-    // With one key block per row the descriptors never change: form them once.  (With more
-    // they are re-formed per stage; that form only serves head dim 8.)
-    Piece fixed[NBLK == 1 ? IPW : 1];
-    if (NBLK == 1) {
+    // The descriptors of a wave's pieces are formed once, for key block 0.  A K, V or mask piece of a later block
+    // lies a fixed number of bytes further on, the same for every lane (K and V: as long as its rows exist; they
+    // are buffer loads there, whose rows at or beyond N read as zero instead of being clamped to the last row).
+    Piece fixed[IPW];
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) fixed[i] = describe(min(wave + 8 * i, I_ALL - 1), 0);
-    }
+    for (int i = 0; i < IPW; ++i) fixed[i] = describe(min(wave + 8 * i, I_ALL - 1), 0);
+    const int kv_valid = (int)(((int64_t)(p.N - 1) * sn + D) * 2);   // bytes from a problem's first K (V) row to the end of its last
+    const int kv_blk = BKV * (int)sn * 2, a_blk = BKV * 16;           // bytes from one key block to the next: K and V rows, mask chunks
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
     // With one stage per row a piece's address is a pointer that all lanes share, advanced by the
     // scalar unit from row to row, plus a 32-bit lane offset that never changes: no 64-bit
     // multiplication per piece and row.  `fnext` is the row the pointers stand at.
-    const unsigned char *fptr[NBLK == 1 ? IPW : 1];
+    const unsigned char *fptr[IPW];
     const float *flse = p.lse + ((int64_t)bh * p.S + s_begin) * p.N;   // of the row the pointers stand at
     const unsigned flse_off = (unsigned)min(qbase + lane, p.N - 1);
-    if (NBLK == 1) {
 #pragma unroll
-        for (int i = 0; i < IPW; ++i) fptr[i] = fixed[i].base;
-    }
-    // moves the pointers from stage t to stage t + 1 (they stay at the last stage)
+    for (int i = 0; i < IPW; ++i) fptr[i] = fixed[i].base;
+    // moves the pointers from stage t to stage t + 1 (they stay at the last stage): to the next S row where
+    // stage t + 1 is a row's first
     auto fetch_advance = [&](int t) {
-        if (NBLK != 1 || t + 1 > T_total - 1) return;
+        if (t + 1 > T_total - 1 || (NBLK != 1 && (t + 1) % NBLK != 0)) return;
 #pragma unroll
         for (int i = 0; i < IPW; ++i) fptr[i] += fixed[i].row_step;
         flse += p.N;
@@ -272,16 +272,22 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             if (NBLK == 1) {
                 stg.v[i] = *reinterpret_cast<const u32x4 *>(fptr[i] + fixed[i].lane_off);
             } else {
-                const Piece d = describe(min(wave + 8 * i, ninst - 1), blk);
-                stg.v[i] = *reinterpret_cast<const u32x4 *>(d.base + row * d.row_step + d.lane_off);
+                const int n = wave + 8 * i;   // uniform
+                if (n < 2 * R::I_K) {
+                    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)fptr[i], 0, kv_valid, 0x00020000);
+                    stg.v[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)fixed[i].lane_off, blk * kv_blk, 0);
+                } else if (n < R::I_KVA) {
+                    stg.v[i] = *reinterpret_cast<const u32x4 *>(fptr[i] + blk * a_blk + fixed[i].lane_off);
+                } else if (blk == 0) {   // (the pieces with query rows belong to a row's first stage)
+                    stg.v[i] = *reinterpret_cast<const u32x4 *>(fptr[i] + fixed[i].lane_off);
+                }
             }
         }
         // the log-sum-exp of the slab's rows travels the same way (one value per lane; every
         // wave asks, wave 0 stores): a load whose result is carried into the next row's
         // prologue in a register would make that prologue wait for everything requested here
-        if (i1 >= IPW) {
-            const int64_t lrow = NBLK == 1 ? 0 : ((int64_t)bh * p.S + s_begin + row) * p.N;
-            const float *lsrc = NBLK == 1 ? flse : p.lse + lrow;
+        if (i1 >= IPW && (NBLK == 1 || blk == 0)) {
+            const float *lsrc = flse;
             stg.lse = lsrc[flse_off];
             // (delta has the layout of the log-sum-exp: the same offset from its own base)
             if (!GATE && e.delta_given) stg.dl = (e.delta + (lsrc - p.lse))[flse_off];
@@ -306,7 +312,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             if (i < i0 || i >= i1) continue;
             const int n = wave + 8 * i;
             if ((NBLK == 1 && 8 * i + 7 < I_ALL) || n < ninst) {
-                const int dst = NBLK == 1 ? fixed[i].dst : describe(n, blk).dst;
+                const int dst = fixed[i].dst;
                 const int qkind = GATE && n >= R::I_KVA ? (n - R::I_KVA) / R::I_Q : -1;   // (GATE: dout, Q, logits, unused, Og)
                 if (n >= 2 * R::I_K && n < R::I_KVA) {   // of a mask chunk (hi, mid, lo, 1, 1, 1, 0, 0) the first 8 bytes
                     *reinterpret_cast<uint2 *>(buf + dst + lane * 8) = make_uint2(stg.v[i][0], stg.v[i][1]);
