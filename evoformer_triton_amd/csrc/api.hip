@@ -517,7 +517,9 @@ int evoattn_bwd(const EvoAttnParams *p0, void *hip_stream) {
     const bool kvring = kv_ring_ok(*p);
     // that kernel sums the dBias partials on its way in (they lie 16-byte aligned for it)
     const bool partials = p->dbias && !dq_writes_dbias(*p);
-    const bool fused_reduce = kvring && partials && !(p->flags & EVO_FLAG_ONLY_DQ) && aligned(p->dbias, 16);
+    // (both dK/dV kernels do; the one-workgroup-per-problem kernel where the sums come in whole 16-byte pieces)
+    const bool fused_reduce = partials && !(p->flags & EVO_FLAG_ONLY_DQ) && aligned(p->dbias, 16) &&
+                              (kvring || ((int64_t)p->B * p->H * p->N * p->N) % 4 == 0);
     e.dbias_chunks = fused_reduce ? e.n_chunks : 0;
     if (p->flags & EVO_FLAG_ONLY_DKDV) return kvring ? launch_mfma_kvr(*p, e, st) : launch_mfma_dkdv(*p, e, st);
     // dQ first: it also writes delta, which the dK/dV kernel reads

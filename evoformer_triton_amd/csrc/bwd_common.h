@@ -85,4 +85,31 @@ static inline int hip_rc() {
     return err == hipSuccess ? EVO_OK : EVO_EHIP - (int)err;
 }
 
+// The dBias partials that the dQ kernel left (one per chunk of its own) summed in chunk order and cast to the dBias
+// dtype, a slice per workgroup, by the dK/dV kernel on its way in: no launch of its own for 16 bytes read per
+// thread and chunk.  Needs B * H * N * N a multiple of 4 and a 16-byte aligned dBias (the caller checks).
+template <int NTH>
+__device__ __forceinline__ void sum_dbias_partials(const EvoAttnParams &p, const Extra &e, int tid) {
+    const int64_t n = (int64_t)p.B * p.H * p.N * p.N;
+    for (int64_t i = ((int64_t)blockIdx.x * NTH + tid) * 4; i < n; i += (int64_t)gridDim.x * NTH * 4) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        for (int c0 = 0; c0 < e.dbias_chunks; c0 += 4) {
+            f32x4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)   // four loads in flight; chunks past the last repeat it and are not added
+                v[j] = *reinterpret_cast<const f32x4 *>(e.dbias_part + (int64_t)min(c0 + j, e.dbias_chunks - 1) * n + i);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (c0 + j < e.dbias_chunks) acc += v[j];
+        }
+        if (p.dbias_dtype == EVO_F32) {
+            *reinterpret_cast<f32x4 *>((float *)p.dbias + i) = acc;
+        } else if (p.dbias_dtype == EVO_BF16) {
+            store4<bf16_t>((bf16_t *)p.dbias + i, acc[0], acc[1], acc[2], acc[3]);
+        } else {
+            store4<f16_t>((f16_t *)p.dbias + i, acc[0], acc[1], acc[2], acc[3]);
+        }
+    }
+}
+
 }  // namespace evo

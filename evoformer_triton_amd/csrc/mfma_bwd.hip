@@ -390,6 +390,9 @@ __global__ void __launch_bounds__(NW * 64, D >= 64 ? 2 : NW == 8 ? 4 : 3) mfma_d
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
 
+    // (where the caller asks for it: the dBias partials summed on the way in, by the workgroups that start first)
+    if (e.dbias_chunks > 0) sum_dbias_partials<NTH>(p, e, tid);
+
     // this wave's keys: requested now, used after the queries have been staged, so that the
     // two round trips to memory overlap
     v8 kraw[KSD], vraw[KSD];

@@ -82,31 +82,9 @@ __global__ void __launch_bounds__(512) mfma_dkdv_ring(EvoAttnParams p, Extra e) 
     const uint2 one3 = ones3<T>();
     const uint2 zero3 = {0u, 0u};
 
-    // The dBias partials that the dQ kernel left (one per chunk of its own) are summed here, in
-    // chunk order, a slice per workgroup, while the first loads of the kernel proper are still
-    // to come: no launch of its own for 16 bytes read per thread and chunk.
-    if (e.dbias_chunks > 0) {
-        const int64_t n = (int64_t)p.B * p.H * p.N * p.N;   // a multiple of 4: N is a multiple of 8
-        for (int64_t i = ((int64_t)blockIdx.x * 512 + tid) * 4; i < n; i += (int64_t)gridDim.x * 512 * 4) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int c0 = 0; c0 < e.dbias_chunks; c0 += 4) {
-                f32x4 v[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)   // four loads in flight; chunks past the last repeat it and are not added
-                    v[j] = *reinterpret_cast<const f32x4 *>(e.dbias_part + (int64_t)min(c0 + j, e.dbias_chunks - 1) * n + i);
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (c0 + j < e.dbias_chunks) acc += v[j];
-            }
-            if (p.dbias_dtype == EVO_F32) {
-                *reinterpret_cast<f32x4 *>((float *)p.dbias + i) = acc;
-            } else if (p.dbias_dtype == EVO_BF16) {
-                store4<bf16_t>((bf16_t *)p.dbias + i, acc[0], acc[1], acc[2], acc[3]);
-            } else {
-                store4<f16_t>((f16_t *)p.dbias + i, acc[0], acc[1], acc[2], acc[3]);
-            }
-        }
-    }
+    // the dBias partials that the dQ kernel left are summed here, a slice per workgroup, while the first loads of the
+    // kernel proper are still to come
+    if (e.dbias_chunks > 0) sum_dbias_partials<512>(p, e, tid);
 
     const int s_begin = c * e.chunk, s_end = min(p.S, s_begin + e.chunk);
     const int nrows = s_end - s_begin;
