@@ -86,8 +86,9 @@ static bool mfma_ok(const EvoAttnParams &p, int pass) {
     if (p.dtype != EVO_BF16 && p.dtype != EVO_F16) return false;
     if (p.D != 8 && p.D != 16 && p.D != 32 && p.D != 64 && p.D != 128) return false;
     if (p.stride_b % 8 || p.stride_h % 8 || p.stride_s % 8 || p.stride_n % 8) return false;
-    // (the forward kernels address the K and V rows of one (b, h, s) problem by 32-bit byte offsets from its first row)
-    if (((int64_t)(p.N - 1) * p.stride_n + p.D) * 2 >= ((int64_t)1 << 31)) return false;
+    // (the kernels address the rows of one (b, h, s) problem by 32-bit byte offsets from its first row, also the rows
+    // up to the next multiple of 256 beyond N, which their buffer loads must find out of range rather than wrapped)
+    if (((int64_t)(p.N + 511) * p.stride_n + p.D) * 2 >= ((int64_t)1 << 31)) return false;
     if (!aligned(p.q, 16) || !aligned(p.k, 16) || !aligned(p.v, 16) || !aligned(p.o, 16)) return false;
     if (pass == EVO_PASS_BWD) {
         if (p.N > 2048 && !long_rows_bwd_ok(p)) return false;

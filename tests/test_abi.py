@@ -58,6 +58,11 @@ def test_check_accepts_a_valid_block(lib):
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
     assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_BWD) == 0
     assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_FWD) == b"mfma"
+    # rows so far apart that a problem's rows (and its padding up to the next 256) leave 32-bit byte offsets: the plain kernels
+    p.stride_n = 1 << 22
+    assert lib.evoattn_check(ctypes.byref(p), _lib.EVO_PASS_FWD) == 0
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_FWD) == b"generic"
+    assert lib.evoattn_path(ctypes.byref(p), _lib.EVO_PASS_BWD) == b"generic"
 
 
 @pytest.mark.parametrize("mutate,code", [
