@@ -37,8 +37,7 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 // QT: 32-row query tiles per workgroup (2, or 1 for rows of several key blocks: half the
 // resident bias tiles and dBias accumulators per wave).
-// KB: keys per stage (256; 128 for head dim 64, whose rows are long, and at head dim 32 for rows of
-// 257..384 keys, which three blocks of 128 cover without an empty half block; 384 for such rows at
+// KB: keys per stage (256; 128 for head dim 64, whose rows are long; 384 for rows of 257..384 keys at
 // head dims 8 and 16, where a whole row fits one stage).
 template <int D, int QT, int KB>
 struct RingGeo {
@@ -106,14 +105,17 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // the dK/dV kernel), dgate = dout * Og * (1 - sigmoid(g)) and delta = rowsum(dO * Og / sigmoid(g)) (to the
 // stage and to e.delta).  Pieces 36..39 are then dout, 40..43 Q, 44..47 the logits, 52..55 Og (a piece and
 // the two that follow it 8 and 16 numbers later belong to the same wave), 48..51 are not used.
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false>
+// LH: the last key block of a row holds at most half a block of keys (rows of 257..384 keys in two blocks of 256): a wave
+// has no tile in its upper half, and keeps neither bias nor dBias sums for one.
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false, bool LH = false>
 __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     typedef Geo<D> G;
     typedef RingGeo<D, QT, KB> R;
     static_assert(R::TPW >= 1 && R::Q_BYTES % 1024 == 0, "query slab too small for this head dim");
     constexpr int KS = G::KS, KSD = G::KSD, DT = G::DT, AUGC = G::AUGC;
     constexpr int C = R::C, BKV = R::BKV, TPB = R::TPB, TPW = R::TPW, RP = R::RP, KQ = R::KQ, QR = R::QR;
-    constexpr int NSLOT = NBLK * TPW;   // key tiles per wave over a whole row
+    static_assert(!LH || (NBLK >= 2 && TPW % 2 == 0), "half a last block needs an even number of tiles per wave and stage");
+    constexpr int NSLOT = NBLK * TPW - (LH ? TPW / 2 : 0);   // key tiles per wave over a whole row
     typedef typename Mfma<T>::v8 v8;
     typedef typename Mfma<T>::v4 v4;
 
@@ -524,6 +526,7 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
             {
 #pragma unroll
                 for (int jj = 0; jj < TPW; ++jj) {
+                    if (LH && blk == NBLK - 1 && jj >= TPW / 2) continue;   // (known at compile time: both loops are unrolled)
                     // The two waves of a SIMD (w and w + 4) take turns at the higher issue priority, tile by tile
                     // (S = 512, N = 256, H = 8, head dim 32: 2 us of 145 less).  Only where a wave has two tiles per
                     // stage: with one, the turn would leave the younger wave ahead throughout, and the older one, which
@@ -678,11 +681,11 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
 
 // ------------------------------------------------------------------ launcher
 
-template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false>
+template <typename T, int D, bool HAS_BIAS, int NBLK, int QT, int KB, bool GATE = false, bool LH = false>
 static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
     typedef RingGeo<D, QT, KB> R;
     static PerDevice done{};
-    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB, GATE>;
+    auto kern = mfma_dq_ring<T, D, HAS_BIAS, NBLK, QT, KB, GATE, LH>;
     if (const int rc = ensure_dynamic_lds((const void *)kern, R::LDS_BYTES, done, nullptr)) return rc;
     const int NT = (p.N + 31) / 32, NQP = (NT + QT - 1) / QT;
     const unsigned grid = (unsigned)NQP * (unsigned)(p.B * p.H) * (unsigned)e.n_chunks;
@@ -699,8 +702,9 @@ static int dqr_launch(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
 //                                         for three blocks of 128 keys, at head dim 8, S = 1024 457 against 467 us for two
 //                                         blocks of 256; at head dim 32 its stage and tiles together spill 113 registers)
 //   head dim 8            N <= 512        2 blocks of 256 keys, 2 query tiles               (4 tiles per wave; its working set is small)
-//   head dim 32           N <= 384        3 blocks of 128 keys, 2 query tiles               (3 tiles per wave; measured
-//                                         196 us against 256 us for the next form at N = 384, D = 32, S = 384, H = 4)
+//   head dim 32           N <= 384        2 blocks of 256 keys, the second at most half full, 2 query tiles (3 tiles per
+//                                         wave, two stages and barriers per row: N = 384, D = 32, S = 384, H = 4 129 us
+//                                         against 142 us for three blocks of 128 keys, the form before)
 //                         N <= 512, 768   2, 3 blocks of 256 keys, 1 query tile             (2, 3 tiles per wave)
 //   head dim 64           N <= 128        1 block of 128 keys, 2 query tiles                (1 tile per wave)
 struct DqrForm {
@@ -711,7 +715,7 @@ constexpr DqrForm dqr_form(int n) {
     if (D == 64) return n <= 128 ? DqrForm{1, 2, 128} : DqrForm{0, 0, 0};
     if (n <= 256) return DqrForm{1, 2, 256};
     if (D == 8) return n <= 384 ? DqrForm{1, 2, 384} : n <= 512 ? DqrForm{2, 2, 256} : DqrForm{0, 0, 0};
-    if (n <= 384) return D == 16 ? DqrForm{1, 2, 384} : DqrForm{3, 2, 128};
+    if (n <= 384) return D == 16 ? DqrForm{1, 2, 384} : DqrForm{2, 2, 256};
     if (n <= 512) return DqrForm{2, 1, 256};
     if (n <= 768) return DqrForm{3, 1, 256};
     return DqrForm{0, 0, 0};
@@ -737,7 +741,7 @@ static int dqr_blocks(const EvoAttnParams &p, const Extra &e, hipStream_t st) {
             if constexpr (D == 16) {
                 if (f.nblk == 1 && f.kb == 384) return dqr_launch<T, D, HAS_BIAS, 1, 2, 384>(p, e, st);
             } else {
-                if (f.nblk == 3 && f.kb == 128) return dqr_launch<T, D, HAS_BIAS, 3, 2, 128>(p, e, st);
+                if (f.nblk == 2 && f.qt == 2) return dqr_launch<T, D, HAS_BIAS, 2, 2, 256, false, true>(p, e, st);
             }
             if (f.nblk == 2) return dqr_launch<T, D, HAS_BIAS, 2, 1, 256>(p, e, st);
             if (f.nblk == 3) return dqr_launch<T, D, HAS_BIAS, 3, 1, 256>(p, e, st);
