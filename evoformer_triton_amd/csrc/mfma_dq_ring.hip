@@ -247,9 +247,9 @@ __global__ void __launch_bounds__(512) mfma_dq_ring(EvoAttnParams p, Extra e) {
     const int kv_blk = BKV * (int)sn * 2, a_blk = BKV * 16;           // bytes from one key block to the next: K and V rows, mask chunks
     // Loads are unconditional (a wave with fewer pieces repeats its last one, the stage past
     // the end repeats the last stage) so that the staging registers stay registers.
-    // With one stage per row a piece's address is a pointer that all lanes share, advanced by the
-    // scalar unit from row to row, plus a 32-bit lane offset that never changes: no 64-bit
-    // multiplication per piece and row.  `fnext` is the row the pointers stand at.
+    // A piece's address is a pointer that all lanes share, advanced by the scalar unit from S row
+    // to S row, plus a 32-bit lane offset that never changes (and, for a later key block of the
+    // row, the block's distance): no 64-bit multiplication per piece and row.
     const unsigned char *fptr[IPW];
     const float *flse = p.lse + ((int64_t)bh * p.S + s_begin) * p.N;   // of the row the pointers stand at
     const unsigned flse_off = (unsigned)min(qbase + lane, p.N - 1);
