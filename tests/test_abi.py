@@ -31,6 +31,15 @@ def test_every_declared_symbol_is_exported(lib):
     assert lib.evoattn_version() == 4
 
 
+def test_the_library_reports_the_version_the_header_declares(lib):
+    text = open(os.path.join(ROOT, "include", "evoattn.h")).read()
+    declared = int(re.search(r"#define\s+EVOATTN_VERSION\s+(\d+)", text).group(1))
+    assert lib.evoattn_version() == declared
+    # (the build entry point checks the same after compiling; it must not carry a number of its own)
+    entry = open(os.path.join(ROOT, "__graft_entry__.py")).read()
+    assert not re.search(r"evoattn_version\(\)\s*==\s*\d", entry)
+
+
 def test_struct_layout_matches_header():
     # 12 x 4-byte fields, 9 x int64, 14 pointers, one size_t, then prep pointer + size; no padding
     assert ctypes.sizeof(EvoAttnParams) == 12 * 4 + 9 * 8 + 14 * 8 + 8 + 16 + 3 * 8        # ... and the three gate pointers
